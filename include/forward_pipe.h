@@ -1,0 +1,149 @@
+// C++ side of the boundary: the abstract network backend the engine programs
+// against, and the two classes this library adds behind it.
+//
+// `ForwardPipe` / `ForwardPipeWeights` re-declare, member for member, the
+// interface of the reference (src/ForwardPipe.h:38-71) so that
+// `Network::init_net` (src/Network.cpp:407-414) can be handed a HIPScheduler
+// where it is handed an OpenCLScheduler today (src/Network.cpp:578-597).
+// Inside the engine the engine's own header is used and `LZHIP_ENGINE_BUILD`
+// makes this file skip the re-declaration.
+#ifndef LZHIP_FORWARD_PIPE_H_INCLUDED
+#define LZHIP_FORWARD_PIPE_H_INCLUDED
+
+#include <atomic>
+#include <condition_variable>
+#include <cstdint>
+#include <deque>
+#include <exception>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "lzhip.h"
+
+#ifndef LZHIP_ENGINE_BUILD
+// Thrown out of forward() when the request was woken by drain()
+// (reference src/Network.h:66-67).
+class NetworkHaltException : public std::exception {};
+
+class ForwardPipe {
+public:
+    // Weights as the network facade hands them over (src/ForwardPipe.h:40-54):
+    // Winograd-domain 3x3 filters, BN means with the conv bias folded in,
+    // BN 1/sqrt(var+eps), and the two 1x1 head convolutions.
+    class ForwardPipeWeights {
+    public:
+        std::vector<std::vector<float>> m_conv_weights;
+        std::vector<std::vector<float>> m_conv_biases;
+        std::vector<std::vector<float>> m_batchnorm_means;
+        std::vector<std::vector<float>> m_batchnorm_stddevs;
+        std::vector<float> m_conv_pol_w;
+        std::vector<float> m_conv_pol_b;
+        std::vector<float> m_conv_val_w;
+        std::vector<float> m_conv_val_b;
+    };
+
+    virtual ~ForwardPipe() = default;
+    virtual void initialize(int channels) = 0;
+    virtual bool needs_autodetect() { return false; }
+    virtual void forward(const std::vector<float>& input, std::vector<float>& output_pol,
+                         std::vector<float>& output_val) = 0;
+    virtual void push_weights(unsigned int filter_size, unsigned int channels,
+                              unsigned int outputs,
+                              std::shared_ptr<const ForwardPipeWeights> weights) = 0;
+    virtual void drain() {}
+    virtual void resume() {}
+};
+#endif  // LZHIP_ENGINE_BUILD
+
+namespace lzhip {
+
+// What the scheduler drives: something that evaluates up to max_batch()
+// positions held in host memory and blocks until the results are back.
+// HIPPipe is the device implementation; the scheduler's unit tests plug in a
+// host-side stand-in so that the queueing logic can run under a thread
+// sanitizer without a GPU.
+class BatchExecutor {
+public:
+    virtual ~BatchExecutor() = default;
+    virtual int max_batch() const = 0;
+    // in [n][18*361] -> pol [n][722], val [n][361]; throws std::runtime_error.
+    virtual void forward_batch(int n, const float* in, float* pol, float* val) = 0;
+};
+
+// Device executor: owns the weights and activation buffers of one network on
+// one GPU and runs the residual tower + 1x1 heads for a batch.  Takes the
+// place of OpenCL<net_t> + OpenCL_Network<net_t> (reference src/OpenCL.h:86-226);
+// there is no tuner, tile shapes are fixed for gfx950.
+class HIPPipe;
+std::unique_ptr<BatchExecutor> make_hip_pipe(int device, int precision, int max_batch,
+                                             int filters);
+
+// Batching scheduler: takes the place of OpenCLScheduler<net_t>
+// (reference src/OpenCLScheduler.h:51-118, .cpp:256-441) for one GPU.
+// Differences that are deliberate:
+//  * a request waits on a per-request done flag (the reference waits on a
+//    condition variable without a predicate, .cpp:272);
+//  * the worker launches whatever is queued, up to max_batch, after a short
+//    adaptive grace period, instead of "full batch or exactly one"
+//    (.cpp:311-353), so that fewer search threads than max_batch still batch.
+class HIPScheduler : public ForwardPipe {
+public:
+    // The engine-facing constructor: device pipe created in initialize().
+    HIPScheduler(int precision, int max_batch, int device = 0);
+    // Test/bring-up constructor: drive an arbitrary executor.
+    explicit HIPScheduler(std::unique_ptr<BatchExecutor> exec);
+    ~HIPScheduler() override;
+
+    void initialize(int channels) override;
+    void forward(const std::vector<float>& input, std::vector<float>& output_pol,
+                 std::vector<float>& output_val) override;
+    void push_weights(unsigned int filter_size, unsigned int channels, unsigned int outputs,
+                      std::shared_ptr<const ForwardPipeWeights> weights) override;
+    void drain() override;
+    void resume() override;
+
+    // Pointer form of forward() used by the C ABI; returns LZHIP_OK/LZHIP_EHALT
+    // and throws std::runtime_error on executor failure.
+    int forward_raw(const float* in, float* pol, float* val);
+
+    BatchExecutor* executor() { return m_exec.get(); }
+    lzhip_stats stats();
+    void reset_stats();
+    // Upper bound, in microseconds, of the grace period the worker grants a
+    // partial batch (0 = launch immediately).
+    void set_max_wait_us(int us);
+
+private:
+    struct Request {
+        const float* in;
+        float* pol;
+        float* val;
+        std::mutex mu;
+        std::condition_variable cv;
+        int state = 0;  // 0 pending, 1 done, 2 halted, 3 failed
+    };
+    void start_worker();
+    void worker();
+
+    int m_precision = LZHIP_FP32, m_max_batch = 1, m_device = 0;
+    std::unique_ptr<BatchExecutor> m_exec;
+    std::mutex m_mutex;
+    std::condition_variable m_cv;
+    std::deque<std::shared_ptr<Request>> m_queue;
+    std::thread m_worker;
+    bool m_running = false;
+    std::atomic<bool> m_draining{false};
+    std::atomic<int> m_outstanding{0};  // callers currently inside forward()
+    int m_max_wait_us = 200;
+    int m_wait_us = 100;
+    std::string* m_fail_msg = nullptr;
+    // statistics
+    std::atomic<uint64_t> m_requests{0}, m_batches{0}, m_halted{0};
+    std::atomic<uint32_t> m_max_seen{0};
+};
+
+}  // namespace lzhip
+#endif

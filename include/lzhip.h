@@ -1,0 +1,180 @@
+/*
+ * lzhip.h -- C ABI of the MI355X (gfx950) network-forward backend for Leela Zero.
+ *
+ * The reference engine has no C ABI of its own: its backends are C++ classes
+ * behind the abstract `ForwardPipe` (reference src/ForwardPipe.h:38-71).  Every
+ * entry point below names the reference interface it stands in for, so that a
+ * maintainer can bind it from the engine (see include/forward_pipe.h for the
+ * C++ classes HIPScheduler / HIPPipe built on the same core).
+ *
+ * Conventions: plain pointers and sizes only; all functions return 0 on success
+ * and a negative LZHIP_E* code on failure; no C++ exception crosses this
+ * boundary; `lzhip_last_error()` returns a thread-local message for the last
+ * failure on the calling thread.  Host pointers unless a name says `_device`.
+ */
+#ifndef LZHIP_H_INCLUDED
+#define LZHIP_H_INCLUDED
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LZHIP_OK 0
+#define LZHIP_EINVAL (-1)   /* bad argument / wrong call order                       */
+#define LZHIP_EDEVICE (-2)  /* HIP runtime error (message in lzhip_last_error)        */
+#define LZHIP_EHALT (-3)    /* request woken by drain(): NetworkHaltException,        */
+                            /* reference src/Network.h:66-67, OpenCLScheduler.cpp:274 */
+#define LZHIP_ENOMEM (-4)
+
+#define LZHIP_FP32 0 /* reference OpenCLScheduler<float>                              */
+#define LZHIP_FP16 1 /* reference OpenCLScheduler<half>: fp16 storage, fp32 accumulate */
+
+/* Fixed sizes of the boundary (reference src/config.h:48-53, src/Network.h:87-91). */
+#define LZHIP_BOARD 19
+#define LZHIP_NPTS 361
+#define LZHIP_INPUT_CHANNELS 18
+#define LZHIP_INPUT_SIZE (18 * 361) /* one position, NCHW, fp32                       */
+#define LZHIP_POL_SIZE (2 * 361)    /* raw policy 1x1-conv planes                     */
+#define LZHIP_VAL_SIZE 361          /* raw value 1x1-conv plane                       */
+#define LZHIP_MOVES 362             /* 361 points + pass                              */
+#define LZHIP_VALUE_LAYER 256
+
+typedef struct lzhip_handle lzhip_handle;
+
+/* Counters of the batching scheduler.  Replaces the reference's debug-only
+ * batch_stats (src/OpenCLScheduler.h:43-49). */
+typedef struct lzhip_stats {
+    uint64_t requests;     /* forward() calls answered with a result                 */
+    uint64_t batches;      /* device batches launched by the scheduler               */
+    uint64_t batch_slots;  /* batches * max_batch : denominator of the fill ratio    */
+    uint64_t halted;       /* forward() calls answered with LZHIP_EHALT              */
+    uint32_t max_batch_seen;
+    uint32_t max_batch;
+} lzhip_stats;
+
+/* ---- life cycle ------------------------------------------------------- */
+
+/* Stands in for constructing the backend + ForwardPipe::initialize(channels)
+ * (reference src/ForwardPipe.h:58, src/OpenCLScheduler.cpp:84-132,
+ * src/Network.cpp:407-414).  `filters` = residual-tower width, `precision` =
+ * LZHIP_FP32 / LZHIP_FP16 (reference cfg_precision, src/GTP.h:104-107),
+ * `max_batch` = reference cfg_batch_size, `device` = HIP device ordinal
+ * (reference --gpu).  Fails with LZHIP_EDEVICE when no gfx950 device or the
+ * HIP runtime is unavailable: there is no CPU fallback. */
+int lzhip_create(int filters, int precision, int max_batch, int device, lzhip_handle** out);
+
+/* Destructor of the backend (reference src/OpenCLScheduler.cpp:134-144):
+ * wakes and joins the worker, pending requests finish with LZHIP_EHALT. */
+int lzhip_destroy(lzhip_handle* h);
+
+/* ForwardPipe::push_weights (reference src/ForwardPipe.h:65-67; contents of
+ * ForwardPipeWeights src/ForwardPipe.h:40-54; call site src/Network.cpp:411).
+ * U[l]        Winograd-domain filters [36][C_in][filters], filters fastest,
+ *             C_in = 18 for l = 0 and `filters` otherwise (src/Network.cpp:215)
+ * bn_mean[l]  [filters], conv bias already folded in   (src/Network.cpp:554-566)
+ * bn_scale[l] [filters], already 1/sqrt(var + 1e-5)    (src/Network.cpp:151-157)
+ * pol_w [2][filters], val_w [filters]  1x1 head convolutions, biases are zero
+ * n_layers = 1 + 2 * residual blocks.  Data is copied; call exactly once. */
+int lzhip_push_weights(lzhip_handle* h, int n_layers, const float* const* U,
+                       const float* const* bn_mean, const float* const* bn_scale,
+                       const float* pol_w, const float* val_w);
+
+/* ---- evaluation ------------------------------------------------------- */
+
+/* ForwardPipe::forward (reference src/ForwardPipe.h:62-64, scheduler
+ * implementation src/OpenCLScheduler.cpp:256-277): one position, blocking,
+ * callable from many threads at once; requests are batched on the device.
+ * in[6498] -> pol[722], val[361] (raw 1x1 outputs, caller-allocated,
+ * src/Network.cpp:819-829).  Returns LZHIP_EHALT if woken by lzhip_drain. */
+int lzhip_forward(lzhip_handle* h, const float* in, float* pol, float* val);
+
+/* Batch executor under the scheduler: OpenCL_Network::forward(batch)
+ * (reference src/OpenCL.cpp:142-329).  n <= max_batch positions, host
+ * buffers, blocking (H2D + tower + 1x1 heads + D2H).  Serialised internally;
+ * does not go through the request queue. */
+int lzhip_forward_batch(lzhip_handle* h, int n, const float* in, float* pol, float* val);
+
+/* Same executor on buffers that already live in device memory (the reference
+ * keeps them in its OpenCLContext, src/OpenCL.h:64-84).  d_in fp32
+ * [n][18][361], d_pol fp32 [n][722], d_val fp32 [n][361].  Enqueues on the
+ * handle's stream and returns without waiting; lzhip_sync waits. */
+int lzhip_forward_batch_device(lzhip_handle* h, int n, const void* d_in, void* d_pol,
+                               void* d_val);
+int lzhip_sync(lzhip_handle* h);
+/* The hipStream_t the handle launches on (for callers that record events). */
+void* lzhip_stream(lzhip_handle* h);
+
+/* ForwardPipe::drain / resume (reference src/ForwardPipe.h:69-70,
+ * src/OpenCLScheduler.cpp:411-441, callers src/UCTSearch.cpp:828-832). */
+int lzhip_drain(lzhip_handle* h);
+int lzhip_resume(lzhip_handle* h);
+
+int lzhip_get_stats(lzhip_handle* h, lzhip_stats* out);
+int lzhip_reset_stats(lzhip_handle* h);
+
+/* ---- heads computed on the device (reference computes them on the host,
+ * src/Network.cpp:833-851) ------------------------------------------------ */
+
+/* Head parameters as Network holds them (reference src/Network.h:166-183),
+ * after the same preprocessing as src/Network.cpp:351-352,568-576:
+ * bn_*_scale = 1/sqrt(var+1e-5), 1x1 conv biases folded into bn_*_mean.
+ * ip_pol_w [362][722], ip1_val_w [256][361], ip2_val_w [256]. */
+int lzhip_push_heads(lzhip_handle* h, const float* bn_pol_mean, const float* bn_pol_scale,
+                     const float* ip_pol_w, const float* ip_pol_b, const float* bn_val_mean,
+                     const float* bn_val_scale, const float* ip1_val_w,
+                     const float* ip1_val_b, const float* ip2_val_w, const float* ip2_val_b);
+
+/* forward_batch + the arithmetic of Network::get_output_internal
+ * (reference src/Network.cpp:833-851, without the symmetry un-rotation):
+ * policy[n][362] = softmax(FC(relu(bn(pol))) / temperature),
+ * value[n] = tanh(FC(relu(FC(relu(bn(val)))))) -- winrate is (1+value)/2.
+ * Optional outputs may be NULL: logits[n][362], pol[n][722], val[n][361]. */
+int lzhip_evaluate_batch(lzhip_handle* h, int n, const float* in, float temperature,
+                         float* policy, float* value, float* logits, float* pol, float* val);
+
+/* ---- weight preparation on the host (no device needed) ----------------- */
+
+/* Network::winograd_transform_f (reference src/Network.cpp:159-223):
+ * f [outputs][channels][3][3] -> U [36][channels][outputs]. */
+int lzhip_winograd_transform_f(const float* f, int outputs, int channels, float* U);
+/* process_bn_var (reference src/Network.cpp:151-157), in place. */
+int lzhip_process_bn_var(float* w, int n);
+
+/* ---- introspection used by the parity tests and the bench --------------- */
+
+/* Runs conv layer `layer` alone on n positions and returns every stage in the
+ * reference's own layouts (src/CPUPipe.cpp:164-174, :196-202, :273-280):
+ * act_in [n][C_in][361] (C_in = 18 for layer 0) -> V [n][36][C_in][25],
+ * M [n][36][filters][25], Y [n][filters][361] after BN (+res) + ReLU.
+ * res [n][filters][361] or NULL.  Activation scaling is off in this call. */
+int lzhip_debug_layer(lzhip_handle* h, int layer, int n, const float* act_in, const float* res,
+                      float* V, float* M, float* Y);
+
+/* Per-layer activation scales chosen for fp16 storage (all 1 in fp32):
+ * out[n_layers + 1]; out[0] is the input scale, out[l + 1] that of layer l. */
+int lzhip_get_act_scales(lzhip_handle* h, float* out, int n);
+
+/* Kernel classes of the tower, for timing. */
+#define LZHIP_K_PACK 0      /* NCHW fp32 input -> channels-last storage type   */
+#define LZHIP_K_IN 1        /* Winograd input transform                        */
+#define LZHIP_K_GEMM 2      /* 36-way batched MFMA GEMM                        */
+#define LZHIP_K_OUT 3       /* output transform + BN + residual + ReLU         */
+#define LZHIP_K_HEAD 4      /* 1x1 policy/value convolutions                   */
+#define LZHIP_K_COUNT 5
+
+/* One forward of n device-resident positions with every kernel launch timed
+ * individually by the device's own begin/end timestamps.  ms[LZHIP_K_COUNT]
+ * receives the summed duration per class, launches[...] the launch counts. */
+int lzhip_profile_forward(lzhip_handle* h, int n, const void* d_in, void* d_pol, void* d_val,
+                          float* ms, int* launches);
+
+const char* lzhip_last_error(void);
+const char* lzhip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

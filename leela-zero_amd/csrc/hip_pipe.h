@@ -1,0 +1,47 @@
+// HIPPipe: the device executor behind the scheduler.  One instance owns the
+// weights, activation buffers and stream of one network on one GPU.
+#pragma once
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "forward_pipe.h"
+
+namespace lzhip {
+
+struct HeadWeightsHost {
+    const float *bn_pol_mean, *bn_pol_scale, *ip_pol_w, *ip_pol_b;
+    const float *bn_val_mean, *bn_val_scale, *ip1_val_w, *ip1_val_b, *ip2_val_w, *ip2_val_b;
+};
+
+class HIPPipe : public BatchExecutor {
+public:
+    ~HIPPipe() override = default;
+
+    // ForwardPipe::push_weights with plain pointers (layouts: include/lzhip.h).
+    virtual void push_weights(int n_layers, const float* const* U, const float* const* bn_mean,
+                              const float* const* bn_scale, const float* pol_w,
+                              const float* val_w) = 0;
+    // Asynchronous forward on device-resident buffers (fp32 in/out).
+    virtual void forward_device(int n, const float* d_in, float* d_pol, float* d_val) = 0;
+    virtual void sync() = 0;
+    virtual void* stream() = 0;
+
+    virtual void push_heads(const HeadWeightsHost& hw) = 0;
+    virtual void evaluate_batch(int n, const float* in, float temperature, float* policy,
+                                float* value, float* logits, float* pol, float* val) = 0;
+
+    virtual void debug_layer(int layer, int n, const float* act_in, const float* res, float* V,
+                             float* M, float* Y) = 0;
+    virtual void profile_forward(int n, const float* d_in, float* d_pol, float* d_val,
+                                 float* ms, int* launches) = 0;
+    virtual std::vector<float> act_scales() const = 0;
+    virtual int filters() const = 0;
+    virtual int precision() const = 0;
+};
+
+// Throws std::runtime_error when the device or runtime is unusable.
+std::unique_ptr<HIPPipe> create_hip_pipe(int device, int precision, int max_batch, int filters);
+
+}  // namespace lzhip

@@ -1,0 +1,289 @@
+// HIPScheduler: request queue + one worker thread that forms batches for the
+// device executor.  Host-only C++ (no HIP calls here), so the queueing logic
+// can be unit-tested on a CPU with a stand-in executor under -fsanitize=thread.
+//
+// Behaviour it keeps from the reference scheduler (src/OpenCLScheduler.cpp):
+//  * forward() blocks the calling search thread until its own result is in
+//    its own buffers (:256-277, :392-403);
+//  * drain() empties the queue and makes every waiting and every later
+//    forward() end with NetworkHaltException until resume() (:411-441);
+//  * the destructor stops the worker and releases waiters (:134-144).
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+
+#include "forward_pipe.h"
+#include "hip_pipe.h"
+
+namespace lzhip {
+
+static constexpr int kInSize = LZHIP_INPUT_SIZE;
+static constexpr int kPolSize = LZHIP_POL_SIZE;
+static constexpr int kValSize = LZHIP_VAL_SIZE;
+
+HIPScheduler::HIPScheduler(int precision, int max_batch, int device)
+    : m_precision(precision), m_max_batch(max_batch), m_device(device) {}
+
+HIPScheduler::HIPScheduler(std::unique_ptr<BatchExecutor> exec) : m_exec(std::move(exec)) {
+    m_max_batch = m_exec->max_batch();
+    start_worker();
+}
+
+HIPScheduler::~HIPScheduler() {
+    {
+        std::lock_guard<std::mutex> lk(m_mutex);
+        m_running = false;
+    }
+    m_cv.notify_all();
+    if (m_worker.joinable()) m_worker.join();
+    // Anything still queued is released as halted.
+    std::deque<std::shared_ptr<Request>> rest;
+    {
+        std::lock_guard<std::mutex> lk(m_mutex);
+        rest.swap(m_queue);
+    }
+    for (auto& r : rest) {
+        {
+            std::lock_guard<std::mutex> lk(r->mu);
+            r->state = 2;
+        }
+        r->cv.notify_all();
+    }
+    delete m_fail_msg;
+}
+
+void HIPScheduler::start_worker() {
+    std::lock_guard<std::mutex> lk(m_mutex);
+    if (m_running) return;
+    m_running = true;
+    m_worker = std::thread(&HIPScheduler::worker, this);
+}
+
+// ForwardPipe::initialize (reference src/OpenCLScheduler.cpp:108-132): create
+// the device pipe for `channels` filters and start the batching worker.
+void HIPScheduler::initialize(int channels) {
+    if (!m_exec) m_exec = make_hip_pipe(m_device, m_precision, m_max_batch, channels);
+    m_max_batch = m_exec->max_batch();
+    start_worker();
+}
+
+// ForwardPipe::push_weights (reference src/OpenCLScheduler.cpp:223-254).
+// filter_size is the Winograd alpha (6) and channels the input plane count
+// (18), as passed by Network::init_net (src/Network.cpp:411).
+void HIPScheduler::push_weights(unsigned int filter_size, unsigned int channels,
+                                unsigned int outputs,
+                                std::shared_ptr<const ForwardPipeWeights> weights) {
+    auto* pipe = dynamic_cast<HIPPipe*>(m_exec.get());
+    if (!pipe) throw std::runtime_error("push_weights: executor is not a device pipe");
+    if (filter_size != 6 || channels != LZHIP_INPUT_CHANNELS)
+        throw std::invalid_argument("push_weights: expected Winograd alpha 6 and 18 input planes");
+    const size_t nl = weights->m_conv_weights.size();
+    if (nl == 0 || weights->m_batchnorm_means.size() != nl ||
+        weights->m_batchnorm_stddevs.size() != nl)
+        throw std::invalid_argument("push_weights: inconsistent layer counts");
+    std::vector<const float*> U(nl), mean(nl), scale(nl);
+    for (size_t l = 0; l < nl; l++) {
+        const size_t cin = l == 0 ? channels : outputs;
+        if (weights->m_conv_weights[l].size() != 36 * cin * outputs ||
+            weights->m_batchnorm_means[l].size() != outputs ||
+            weights->m_batchnorm_stddevs[l].size() != outputs)
+            throw std::invalid_argument("push_weights: layer has the wrong size");
+        U[l] = weights->m_conv_weights[l].data();
+        mean[l] = weights->m_batchnorm_means[l].data();
+        scale[l] = weights->m_batchnorm_stddevs[l].data();
+    }
+    if (weights->m_conv_pol_w.size() != 2 * (size_t)outputs ||
+        weights->m_conv_val_w.size() != (size_t)outputs)
+        throw std::invalid_argument("push_weights: head convolutions have the wrong size");
+    pipe->push_weights((int)nl, U.data(), mean.data(), scale.data(),
+                       weights->m_conv_pol_w.data(), weights->m_conv_val_w.data());
+}
+
+void HIPScheduler::forward(const std::vector<float>& input, std::vector<float>& output_pol,
+                           std::vector<float>& output_val) {
+    if (input.size() != (size_t)kInSize || output_pol.size() != (size_t)kPolSize ||
+        output_val.size() != (size_t)kValSize)
+        throw std::invalid_argument("forward: wrong vector sizes");
+    if (forward_raw(input.data(), output_pol.data(), output_val.data()) == LZHIP_EHALT)
+        throw NetworkHaltException();
+}
+
+int HIPScheduler::forward_raw(const float* in, float* pol, float* val) {
+    if (m_draining.load()) {
+        m_halted++;
+        return LZHIP_EHALT;
+    }
+    auto req = std::make_shared<Request>();
+    req->in = in;
+    req->pol = pol;
+    req->val = val;
+    m_outstanding++;
+    {
+        std::lock_guard<std::mutex> lk(m_mutex);
+        if (!m_running) {
+            m_outstanding--;
+            throw std::runtime_error("forward: scheduler is not initialised");
+        }
+        // drain() may have started between the check above and here
+        if (m_draining.load()) {
+            m_outstanding--;
+            m_halted++;
+            return LZHIP_EHALT;
+        }
+        m_queue.push_back(req);
+    }
+    m_cv.notify_one();
+    int state;
+    {
+        std::unique_lock<std::mutex> lk(req->mu);
+        req->cv.wait(lk, [&] { return req->state != 0; });
+        state = req->state;
+    }
+    m_outstanding--;
+    if (state == 1) {
+        m_requests++;
+        return LZHIP_OK;
+    }
+    if (state == 2) {
+        m_halted++;
+        return LZHIP_EHALT;
+    }
+    std::string msg;
+    {
+        std::lock_guard<std::mutex> lk(m_mutex);
+        msg = m_fail_msg ? *m_fail_msg : std::string("executor failure");
+    }
+    throw std::runtime_error(msg);
+}
+
+// Batch pickup.  The worker sleeps until a request exists, then grants a
+// short grace period for the batch to grow towards the number of callers
+// that are currently inside forward() (they cannot all be queued yet when the
+// first one arrives).  The grace period adapts: it shrinks when it expired
+// without the batch growing and grows, up to m_max_wait_us, when requests
+// kept arriving during it.
+void HIPScheduler::worker() {
+    std::vector<float> in, pol, val;
+    in.resize((size_t)m_max_batch * kInSize);
+    pol.resize((size_t)m_max_batch * kPolSize);
+    val.resize((size_t)m_max_batch * kValSize);
+    std::vector<std::shared_ptr<Request>> batch;
+    for (;;) {
+        batch.clear();
+        {
+            std::unique_lock<std::mutex> lk(m_mutex);
+            m_cv.wait(lk, [&] { return !m_running || !m_queue.empty(); });
+            if (!m_running) return;
+            const auto want = [&]() -> size_t {
+                const int o = m_outstanding.load();
+                return (size_t)std::max(1, std::min(m_max_batch, o));
+            };
+            if (m_queue.size() < want() && m_max_wait_us > 0) {
+                const size_t before = m_queue.size();
+                const auto deadline =
+                    std::chrono::steady_clock::now() + std::chrono::microseconds(m_wait_us);
+                m_cv.wait_until(lk, deadline, [&] {
+                    return !m_running || m_queue.empty() || m_queue.size() >= want();
+                });
+                if (!m_running) return;
+                if (m_queue.size() < want()) {
+                    if (m_queue.size() > before)
+                        m_wait_us = std::min(m_max_wait_us, m_wait_us * 2 + 1);
+                    else
+                        m_wait_us = std::max(1, m_wait_us / 2);
+                }
+            }
+            // drain() may have emptied the queue while we waited
+            while (!m_queue.empty() && (int)batch.size() < m_max_batch) {
+                batch.push_back(std::move(m_queue.front()));
+                m_queue.pop_front();
+            }
+        }
+        if (batch.empty()) continue;
+        const int n = (int)batch.size();
+        for (int i = 0; i < n; i++)
+            std::memcpy(in.data() + (size_t)i * kInSize, batch[i]->in, sizeof(float) * kInSize);
+        int outcome = 1;
+        try {
+            m_exec->forward_batch(n, in.data(), pol.data(), val.data());
+        } catch (const std::exception& e) {
+            outcome = 3;
+            std::lock_guard<std::mutex> lk(m_mutex);
+            delete m_fail_msg;
+            m_fail_msg = new std::string(e.what());
+        }
+        m_batches++;
+        uint32_t seen = m_max_seen.load();
+        while ((uint32_t)n > seen && !m_max_seen.compare_exchange_weak(seen, (uint32_t)n)) {}
+        for (int i = 0; i < n; i++) {
+            Request& r = *batch[i];
+            if (outcome == 1) {
+                std::memcpy(r.pol, pol.data() + (size_t)i * kPolSize, sizeof(float) * kPolSize);
+                std::memcpy(r.val, val.data() + (size_t)i * kValSize, sizeof(float) * kValSize);
+            }
+            {
+                std::lock_guard<std::mutex> lk(r.mu);
+                r.state = outcome;
+            }
+            r.cv.notify_all();
+        }
+    }
+}
+
+// ForwardPipe::drain (reference src/OpenCLScheduler.cpp:411-433): requests
+// still queued are released as halted; a batch already on the device
+// completes normally.
+void HIPScheduler::drain() {
+    m_draining.store(true);
+    std::deque<std::shared_ptr<Request>> taken;
+    {
+        std::lock_guard<std::mutex> lk(m_mutex);
+        taken.swap(m_queue);
+    }
+    m_cv.notify_all();
+    for (auto& r : taken) {
+        {
+            std::lock_guard<std::mutex> lk(r->mu);
+            r->state = 2;
+        }
+        r->cv.notify_all();
+    }
+}
+
+// ForwardPipe::resume (reference src/OpenCLScheduler.cpp:435-441).  The
+// caller has joined its search threads, so the queue is empty.
+void HIPScheduler::resume() {
+    {
+        std::lock_guard<std::mutex> lk(m_mutex);
+        if (!m_queue.empty()) throw std::logic_error("resume: requests are still queued");
+    }
+    m_draining.store(false);
+}
+
+void HIPScheduler::set_max_wait_us(int us) {
+    std::lock_guard<std::mutex> lk(m_mutex);
+    m_max_wait_us = std::max(0, us);
+    m_wait_us = std::max(1, std::min(m_wait_us, std::max(1, m_max_wait_us)));
+}
+
+lzhip_stats HIPScheduler::stats() {
+    lzhip_stats s;
+    s.requests = m_requests.load();
+    s.batches = m_batches.load();
+    s.batch_slots = s.batches * (uint64_t)m_max_batch;
+    s.halted = m_halted.load();
+    s.max_batch_seen = m_max_seen.load();
+    s.max_batch = (uint32_t)m_max_batch;
+    return s;
+}
+
+void HIPScheduler::reset_stats() {
+    m_requests = 0;
+    m_batches = 0;
+    m_halted = 0;
+    m_max_seen = 0;
+}
+
+}  // namespace lzhip

@@ -1,0 +1,70 @@
+// Launch interface of the gfx950 kernels of the residual tower.
+//
+// Device data layouts (P = storage type: float or _Float16):
+//   act  [n][361][Cp]        activations, channels fastest ("channels-last")
+//   V    [36][Tp][Cp]        Winograd-domain input tiles, t = board*25 + by*5 + bx
+//   U    [36][Kp][Cp]        Winograd-domain filters, input channel fastest
+//   M    [36][Tp][Kp]        per-position GEMM results, output channel fastest
+// Cp, Kp are the channel counts padded to a multiple of 64, Tp the tile count
+// padded to a multiple of 128.  The contraction index (input channel) is the
+// fastest-moving one of both GEMM operands, which is what the MFMA operand
+// registers want: each lane fetches 16 contiguous bytes of one row.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace lzhip {
+
+constexpr int kBoard = 19;
+constexpr int kPts = 361;
+constexpr int kTilesPerBoard = 25;
+constexpr int kPos = 36;       // 6x6 Winograd positions
+constexpr int kInPlanes = 18;
+constexpr int kGemmBM = 128;   // GEMM tile extent along T; Tp is a multiple of it
+
+// Timing hook: when non-null every launch is bracketed by this event pair
+// (device begin/end timestamps of that launch alone).
+struct LaunchTimer {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+
+// NCHW fp32 planes [n][C][361] -> act [n][361][Cp] (channels >= C zero).
+template <typename P>
+void launch_pack_input(const float* in, P* act, int n, int C, int Cp, hipStream_t s,
+                       LaunchTimer* t);
+
+// act [n][361][Cp] -> V [36][Tp][Cp]
+template <typename P>
+void launch_in_transform(const P* act, P* V, int n, int Cp, int Tp, hipStream_t s,
+                         LaunchTimer* t);
+
+// M[p][t][k] = sum_c V[p][t][c] * U[p][k][c]
+template <typename P>
+void launch_gemm(const P* V, const P* U, P* M, int Tp_used, int Tp, int Cp, int Kp,
+                 hipStream_t s, LaunchTimer* t);
+
+// M [36][Tp][Kp] -> out [n][361][Kp]:  max(0, scale*(A^T m A - mean) + rfac*res)
+template <typename P>
+void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scale,
+                          const float* bn_mean, float rfac, int n, int Kp, int Tp,
+                          hipStream_t s, LaunchTimer* t);
+
+// 1x1 head convolutions: act [n][361][Cp] x w[3][Cp] -> pol [n][2][361], val [n][361],
+// both multiplied by out_scale.
+template <typename P>
+void launch_head_conv(const P* act, const float* w3, float out_scale, float* pol, float* val,
+                      int n, int Cp, hipStream_t s, LaunchTimer* t);
+
+// max |x| over count elements -> *out (float, must be zeroed before).
+template <typename P>
+void launch_absmax(const P* x, size_t count, float* out, hipStream_t s);
+
+// Head arithmetic above the pipe boundary, one workgroup per position.
+struct HeadParams {
+    const float *bn_pol_mean, *bn_pol_scale, *ip_pol_w, *ip_pol_b;
+    const float *bn_val_mean, *bn_val_scale, *ip1_val_w, *ip1_val_b, *ip2_val_w, *ip2_val_b;
+};
+void launch_heads(const float* pol, const float* val, HeadParams hp, float temperature,
+                  float* policy, float* logits, float* value, int n, hipStream_t s);
+
+}  // namespace lzhip

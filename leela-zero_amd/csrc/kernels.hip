@@ -1,0 +1,599 @@
+// gfx950 (CDNA4) kernels of the Winograd F(4x4,3x3) residual tower.
+//
+// Arithmetic follows the reference CPU pipe (reference src/CPUPipe.cpp:63-284,
+// :352-377) and its OpenCL twins (src/kernels/convolve3.opencl:47-79); the
+// decomposition, layouts and launch shapes are this library's own.
+#include "kernels.h"
+
+#include <hip/hip_ext.h>
+
+namespace lzhip {
+
+typedef _Float16 half_t;
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+#define SQ2 1.4142135623730951f
+
+// ---------------------------------------------------------------------------
+// Per-lane channel vector: how many consecutive channels one lane owns in the
+// bandwidth-bound kernels (4 bytes per lane and access for both types).
+template <typename P> struct ChanVec;
+template <> struct ChanVec<float> {
+    static constexpr int N = 1;
+    static __device__ __forceinline__ void load(const float* p, float* o) { o[0] = *p; }
+    static __device__ __forceinline__ void store(float* p, const float* v) { *p = v[0]; }
+};
+template <> struct ChanVec<half_t> {
+    static constexpr int N = 2;
+    static __device__ __forceinline__ void load(const half_t* p, float* o) {
+        const half2v h = *reinterpret_cast<const half2v*>(p);
+        o[0] = (float)h.x;
+        o[1] = (float)h.y;
+    }
+    // Saturating: a value beyond the fp16 range is stored as +-65504, not inf.
+    static __device__ __forceinline__ void store(half_t* p, const float* v) {
+        half2v h;
+        h.x = (half_t)fminf(fmaxf(v[0], -65504.0f), 65504.0f);
+        h.y = (half_t)fminf(fmaxf(v[1], -65504.0f), 65504.0f);
+        *reinterpret_cast<half2v*>(p) = h;
+    }
+};
+
+template <typename P> __device__ __forceinline__ P to_storage(float v);
+template <> __device__ __forceinline__ float to_storage<float>(float v) { return v; }
+template <> __device__ __forceinline__ half_t to_storage<half_t>(float v) {
+    return (half_t)fminf(fmaxf(v, -65504.0f), 65504.0f);
+}
+
+// o = B^T i for one 6-vector (reference src/CPUPipe.cpp:88-106).
+__device__ __forceinline__ void bt6(const float i0, const float i1, const float i2,
+                                    const float i3, const float i4, const float i5, float& o0,
+                                    float& o1, float& o2, float& o3, float& o4, float& o5) {
+    const float a = i1 * -SQ2 + i3 * (SQ2 / 2.0f);
+    const float b = i2 * -2.0f + i4;
+    o0 = i0 + i2 * (-5.0f / 2.0f) + i4;
+    o1 = a + b;
+    o2 = -a + b;
+    const float c = i3 * SQ2 + i1 * (-SQ2 / 2.0f);
+    const float d = i2 * (-1.0f / 2.0f) + i4;
+    o3 = c + d;
+    o4 = -c + d;
+    o5 = i1 + i3 * (-5.0f / 2.0f) + i5;
+}
+
+// o = A^T i for one 6-vector (reference src/CPUPipe.cpp:225-238).
+__device__ __forceinline__ void at6(const float i0, const float i1, const float i2,
+                                    const float i3, const float i4, const float i5, float& o0,
+                                    float& o1, float& o2, float& o3) {
+    const float t1p2 = (i1 + i2) * (1.0f / 2.0f);
+    const float t1m2 = (i1 - i2) * (SQ2 / 4.0f);
+    const float t3p4 = i3 + i4;
+    const float t3m4 = (i3 - i4) * SQ2;
+    o0 = i0 + t1p2 + t1p2 + t3p4;
+    o1 = t1m2 + t1m2 + t3m4;
+    o2 = t1p2 + t3p4 + t3p4;
+    o3 = t1m2 + t3m4 + t3m4 + i5;
+}
+
+// ---------------------------------------------------------------------------
+template <typename K, typename... Args>
+static inline void launch(K kernel, dim3 grid, dim3 block, hipStream_t s, LaunchTimer* t,
+                          Args... args) {
+    if (t && t->start) {
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, s, t->start, t->stop, 0, args...);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, 0, s, args...);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Planes NCHW fp32 [n][C][361] -> channels-last storage type [n][361][Cp],
+// channels C..Cp-1 zero.
+template <typename P>
+__global__ __launch_bounds__(256) void pack_input_k(const float* __restrict__ in,
+                                                    P* __restrict__ act, int n, int C, int Cp) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t total = (size_t)n * kPts * Cp;
+    if (gid >= total) return;
+    const int c = (int)(gid % Cp);
+    const size_t bp = gid / Cp;
+    const int pt = (int)(bp % kPts);
+    const size_t b = bp / kPts;
+    float v = 0.0f;
+    if (c < C) v = in[(b * C + c) * kPts + pt];
+    act[gid] = to_storage<P>(v);
+}
+
+template <typename P>
+void launch_pack_input(const float* in, P* act, int n, int C, int Cp, hipStream_t s,
+                       LaunchTimer* t) {
+    const size_t total = (size_t)n * kPts * Cp;
+    launch(pack_input_k<P>, dim3((unsigned)((total + 255) / 256)), dim3(256), s, t, in, act, n, C,
+           Cp);
+}
+
+// ---------------------------------------------------------------------------
+// Winograd input transform V = B^T d B (reference src/CPUPipe.cpp:63-183).
+// One lane owns one tile and ChanVec<P>::N consecutive channels; consecutive
+// lanes own consecutive channels, so every load and store of a wave covers a
+// contiguous run of the channels-last arrays.  The 6x6 patch starts one point
+// above/left of board point (4by, 4bx); points off the board read as zero.
+template <typename P>
+__global__ __launch_bounds__(256) void in_transform_k(const P* __restrict__ act,
+                                                      P* __restrict__ V, int T, int Cp,
+                                                      int Tp) {
+    constexpr int VN = ChanVec<P>::N;
+    const int lpt = Cp / VN;  // lanes per tile
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int t = gid / lpt;
+    if (t >= T) return;
+    const int c = (gid - t * lpt) * VN;
+    const int b = t / kTilesPerBoard;
+    const int j = t - b * kTilesPerBoard;
+    const int by = j / 5, bx = j - by * 5;
+    const int y0 = 4 * by - 1, x0 = 4 * bx - 1;
+    const P* base = act + (size_t)b * kPts * Cp + c;
+
+    float d[VN][36];
+#pragma unroll
+    for (int yy = 0; yy < 6; yy++) {
+#pragma unroll
+        for (int xx = 0; xx < 6; xx++) {
+            const int y = y0 + yy, x = x0 + xx;
+            float tmp[VN];
+#pragma unroll
+            for (int v = 0; v < VN; v++) tmp[v] = 0.0f;
+            if ((unsigned)y < (unsigned)kBoard && (unsigned)x < (unsigned)kBoard)
+                ChanVec<P>::load(base + (size_t)(y * kBoard + x) * Cp, tmp);
+#pragma unroll
+            for (int v = 0; v < VN; v++) d[v][yy * 6 + xx] = tmp[v];
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VN; v++) {
+        float t1[36];
+#pragma unroll
+        for (int xx = 0; xx < 6; xx++)  // columns: along y
+            bt6(d[v][0 + xx], d[v][6 + xx], d[v][12 + xx], d[v][18 + xx], d[v][24 + xx],
+                d[v][30 + xx], t1[0 + xx], t1[6 + xx], t1[12 + xx], t1[18 + xx], t1[24 + xx],
+                t1[30 + xx]);
+#pragma unroll
+        for (int yy = 0; yy < 6; yy++)  // rows: along x
+            bt6(t1[yy * 6 + 0], t1[yy * 6 + 1], t1[yy * 6 + 2], t1[yy * 6 + 3], t1[yy * 6 + 4],
+                t1[yy * 6 + 5], d[v][yy * 6 + 0], d[v][yy * 6 + 1], d[v][yy * 6 + 2],
+                d[v][yy * 6 + 3], d[v][yy * 6 + 4], d[v][yy * 6 + 5]);
+    }
+    P* vout = V + (size_t)t * Cp + c;
+    const size_t pstride = (size_t)Tp * Cp;
+#pragma unroll
+    for (int p = 0; p < 36; p++) {
+        float tmp[VN];
+#pragma unroll
+        for (int v = 0; v < VN; v++) tmp[v] = d[v][p];
+        ChanVec<P>::store(vout + p * pstride, tmp);
+    }
+}
+
+template <typename P>
+void launch_in_transform(const P* act, P* V, int n, int Cp, int Tp, hipStream_t s,
+                         LaunchTimer* t) {
+    const int T = n * kTilesPerBoard;
+    const int lanes = T * (Cp / ChanVec<P>::N);
+    launch(in_transform_k<P>, dim3((lanes + 255) / 256), dim3(256), s, t, act, V, T, Cp, Tp);
+}
+
+// ---------------------------------------------------------------------------
+// Output transform Y = A^T m A fused with batch-norm scale/shift, residual add
+// and ReLU (reference src/CPUPipe.cpp:212-284 + :352-377; the reference GPU
+// path fuses the same way, src/kernels/convolve3.opencl:218-318).
+// out = max(0, scale*(y - mean) + rfac*res); rfac carries the ratio of the
+// activation scales of the skip connection and of this layer (1 in fp32).
+template <typename P>
+__global__ __launch_bounds__(256) void out_transform_k(
+    const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ out,
+    const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int T,
+    int Kp, int Tp) {
+    constexpr int VN = ChanVec<P>::N;
+    const int lpt = Kp / VN;
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int t = gid / lpt;
+    if (t >= T) return;
+    const int c = (gid - t * lpt) * VN;
+    const int b = t / kTilesPerBoard;
+    const int j = t - b * kTilesPerBoard;
+    const int by = j / 5, bx = j - by * 5;
+
+    float m[VN][36];
+    const P* min = M + (size_t)t * Kp + c;
+    const size_t pstride = (size_t)Tp * Kp;
+#pragma unroll
+    for (int p = 0; p < 36; p++) {
+        float tmp[VN];
+        ChanVec<P>::load(min + p * pstride, tmp);
+#pragma unroll
+        for (int v = 0; v < VN; v++) m[v][p] = tmp[v];
+    }
+    float o[VN][16];
+#pragma unroll
+    for (int v = 0; v < VN; v++) {
+        float t1[24];  // [4][6]
+#pragma unroll
+        for (int xx = 0; xx < 6; xx++)
+            at6(m[v][0 + xx], m[v][6 + xx], m[v][12 + xx], m[v][18 + xx], m[v][24 + xx],
+                m[v][30 + xx], t1[0 + xx], t1[6 + xx], t1[12 + xx], t1[18 + xx]);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            at6(t1[i * 6 + 0], t1[i * 6 + 1], t1[i * 6 + 2], t1[i * 6 + 3], t1[i * 6 + 4],
+                t1[i * 6 + 5], o[v][i * 4 + 0], o[v][i * 4 + 1], o[v][i * 4 + 2],
+                o[v][i * 4 + 3]);
+    }
+    float sc[VN], mn[VN];
+#pragma unroll
+    for (int v = 0; v < VN; v++) {
+        sc[v] = bn_scale[c + v];
+        mn[v] = bn_mean[c + v];
+    }
+    const size_t bbase = (size_t)b * kPts * Kp + c;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const int y = 4 * by + i, x = 4 * bx + jj;
+            if (y < kBoard && x < kBoard) {
+                const size_t idx = bbase + (size_t)(y * kBoard + x) * Kp;
+                float val[VN];
+#pragma unroll
+                for (int v = 0; v < VN; v++) val[v] = sc[v] * (o[v][i * 4 + jj] - mn[v]);
+                if (res != nullptr) {
+                    float r[VN];
+                    ChanVec<P>::load(res + idx, r);
+#pragma unroll
+                    for (int v = 0; v < VN; v++) val[v] = val[v] + rfac * r[v];
+                }
+#pragma unroll
+                for (int v = 0; v < VN; v++) val[v] = fmaxf(0.0f, val[v]);
+                ChanVec<P>::store(out + idx, val);
+            }
+        }
+    }
+}
+
+template <typename P>
+void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scale,
+                          const float* bn_mean, float rfac, int n, int Kp, int Tp,
+                          hipStream_t s, LaunchTimer* t) {
+    const int T = n * kTilesPerBoard;
+    const int lanes = T * (Kp / ChanVec<P>::N);
+    launch(out_transform_k<P>, dim3((lanes + 255) / 256), dim3(256), s, t, M, res, out,
+           bn_scale, bn_mean, rfac, T, Kp, Tp);
+}
+
+// ---------------------------------------------------------------------------
+// The 36 independent GEMMs M_p[t][k] = sum_c V_p[t][c] * U_p[k][c]
+// (reference src/CPUPipe.cpp:185-210; GPU twin XgemmBatched).
+//
+// One workgroup = 4 wavefronts (2x2) computes a BM x BN tile of one position.
+// Both operands are staged through LDS in 128-byte-per-row slices (64 halves
+// or 32 floats of the contraction index), double buffered, rows padded by 16
+// bytes so that the 16-byte-per-lane fragment reads are conflict free.
+// Each lane feeds the matrix cores with 16 contiguous bytes of its row:
+//   fp16: one v_mfma_f32_32x32x16_f16 per fragment pair (8 halves per lane)
+//   fp32: four v_mfma_f32_32x32x2_f32 per fragment pair (one float each)
+// Lane l supplies row (l & 31) of the A block / column (l & 31) of the B
+// block, and the upper half-wave supplies the other half of the k-slice; the
+// assignment of k values to MFMA k-slots is the same for A and B, which is
+// all the contraction needs.  Accumulation is fp32 for both storage types.
+template <typename P> struct Mma;
+template <> struct Mma<half_t> {
+    static __device__ __forceinline__ float16v run(int4v a, int4v b, float16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, a),
+                                                      __builtin_bit_cast(half8v, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mma<float> {
+    static __device__ __forceinline__ float16v run(int4v a, int4v b, float16v c) {
+        const float4v fa = __builtin_bit_cast(float4v, a);
+        const float4v fb = __builtin_bit_cast(float4v, b);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.x, fb.x, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.y, fb.y, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.z, fb.z, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.w, fb.w, c, 0, 0, 0);
+        return c;
+    }
+};
+
+template <typename P, int BM, int BN>
+__global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
+                                                   const P* __restrict__ U, P* __restrict__ M,
+                                                   int Tp, int Cp, int Kp, int tiles_m,
+                                                   int tiles_n) {
+    constexpr int EPC = 16 / sizeof(P);   // elements per 16-byte chunk
+    constexpr int BK = 128 / sizeof(P);   // contraction extent of one LDS stage
+    constexpr int ROW = BK + EPC;         // padded LDS row, in elements (144 bytes)
+    constexpr int WM = BM / 2, WN = BN / 2;
+    constexpr int MB = WM / 32, NB = WN / 32;
+    constexpr int A_CH = BM * 8 / 256, B_CH = BN * 8 / 256;  // chunks per thread and stage
+    static_assert(MB >= 1 && NB >= 1, "tile too small for a 2x2 wave grid");
+
+    __shared__ __attribute__((aligned(16))) P As[2][BM * ROW];
+    __shared__ __attribute__((aligned(16))) P Bs[2][BN * ROW];
+
+    int bid = blockIdx.x;
+    const int tn = bid % tiles_n;
+    bid /= tiles_n;
+    const int tm = bid % tiles_m;
+    const int p = bid / tiles_m;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wy = wave >> 1, wx = wave & 1;
+    const P* Ag = V + ((size_t)p * Tp + (size_t)tm * BM) * Cp;
+    const P* Bg = U + ((size_t)p * Kp + (size_t)tn * BN) * Cp;
+
+    float16v acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    int4v ra[A_CH], rb[B_CH];
+    const int lrow = tid >> 3, lch = tid & 7;  // row / chunk of this thread's first chunk
+
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_CH; i++)
+            ra[i] = *reinterpret_cast<const int4v*>(Ag + (size_t)(lrow + i * 32) * Cp + k0 +
+                                                    lch * EPC);
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+            rb[i] = *reinterpret_cast<const int4v*>(Bg + (size_t)(lrow + i * 32) * Cp + k0 +
+                                                    lch * EPC);
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_CH; i++)
+            *reinterpret_cast<int4v*>(&As[buf][(lrow + i * 32) * ROW + lch * EPC]) = ra[i];
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+            *reinterpret_cast<int4v*>(&Bs[buf][(lrow + i * 32) * ROW + lch * EPC]) = rb[i];
+    };
+
+    const int nk = Cp / BK;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+
+    const int frow = lane & 31, fk = (lane >> 5) * EPC;
+    for (int kt = 0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) gload((kt + 1) * BK);
+#pragma unroll
+        for (int kc = 0; kc < 4; kc++) {
+            int4v fa[MB], fb[NB];
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+                fa[i] = *reinterpret_cast<const int4v*>(
+                    &As[cur][(wy * WM + i * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                fb[j] = *reinterpret_cast<const int4v*>(
+                    &Bs[cur][(wx * WN + j * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++) acc[i][j] = Mma<P>::run(fa[i], fb[j], acc[i][j]);
+        }
+        if (kt + 1 < nk) lstore(cur ^ 1);
+        __syncthreads();
+    }
+
+    // Accumulator layout of the 32x32 MFMA: register r of lane l holds
+    // row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+    P* Mg = M + ((size_t)p * Tp + (size_t)tm * BM + wy * WM) * Kp + (size_t)tn * BN + wx * WN;
+    const int crow = 4 * (lane >> 5), ccol = lane & 31;
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = i * 32 + 8 * (r >> 2) + crow + (r & 3);
+                Mg[(size_t)row * Kp + j * 32 + ccol] = to_storage<P>(acc[i][j][r]);
+            }
+}
+
+template <typename P>
+void launch_gemm(const P* V, const P* U, P* M, int Tp_used, int Tp, int Cp, int Kp,
+                 hipStream_t s, LaunchTimer* t) {
+    const int tiles_m = Tp_used / kGemmBM;
+    if (Kp % 128 == 0) {
+        const int tiles_n = Kp / 128;
+        launch(wino_gemm_k<P, kGemmBM, 128>, dim3(tiles_m * tiles_n * kPos), dim3(256), s, t, V,
+               U, M, Tp, Cp, Kp, tiles_m, tiles_n);
+    } else {
+        const int tiles_n = Kp / 64;
+        launch(wino_gemm_k<P, kGemmBM, 64>, dim3(tiles_m * tiles_n * kPos), dim3(256), s, t, V,
+               U, M, Tp, Cp, Kp, tiles_m, tiles_n);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// 1x1 policy (2 planes) and value (1 plane) convolutions in one pass over the
+// last activation (reference src/CPUPipe.cpp:424-427).  One wavefront per
+// board point; lanes stride over channels, then a butterfly reduction.
+template <typename P>
+__global__ __launch_bounds__(256) void head_conv_k(const P* __restrict__ act,
+                                                   const float* __restrict__ w3,
+                                                   float out_scale, float* __restrict__ pol,
+                                                   float* __restrict__ val, int n, int Cp) {
+    const int gw = (blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    if (gw >= n * kPts) return;
+    const int b = gw / kPts, pt = gw - b * kPts;
+    const P* a = act + (size_t)gw * Cp;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    for (int c = lane; c < Cp; c += 64) {
+        const float x = (float)a[c];
+        s0 += x * w3[c];
+        s1 += x * w3[Cp + c];
+        s2 += x * w3[2 * Cp + c];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        s0 += __shfl_xor(s0, off);
+        s1 += __shfl_xor(s1, off);
+        s2 += __shfl_xor(s2, off);
+    }
+    if (lane == 0) {
+        pol[(size_t)b * 2 * kPts + pt] = s0 * out_scale;
+        pol[(size_t)b * 2 * kPts + kPts + pt] = s1 * out_scale;
+        val[(size_t)b * kPts + pt] = s2 * out_scale;
+    }
+}
+
+template <typename P>
+void launch_head_conv(const P* act, const float* w3, float out_scale, float* pol, float* val,
+                      int n, int Cp, hipStream_t s, LaunchTimer* t) {
+    const int waves = n * kPts;
+    launch(head_conv_k<P>, dim3((waves + 3) / 4), dim3(256), s, t, act, w3, out_scale, pol, val,
+           n, Cp);
+}
+
+// ---------------------------------------------------------------------------
+template <typename P>
+__global__ __launch_bounds__(256) void absmax_k(const P* __restrict__ x, size_t count,
+                                                float* out) {
+    float m = 0.0f;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count;
+         i += (size_t)gridDim.x * 256) {
+        const float v = fabsf((float)x[i]);
+        // NaN-propagating max so that a poisoned buffer is visible to the host.
+        m = (v != v) ? INFINITY : fmaxf(m, v);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if ((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<int*>(out), __float_as_int(m));
+}
+
+template <typename P>
+void launch_absmax(const P* x, size_t count, float* out, hipStream_t s) {
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(absmax_k<P>, dim3((unsigned)blocks), dim3(256), 0, s, x, count, out);
+}
+
+// ---------------------------------------------------------------------------
+// Head arithmetic above the pipe boundary (reference src/Network.cpp:833-851):
+// policy: BN+ReLU on 2 planes -> FC 722->362 -> softmax(./temperature)
+// value : BN+ReLU on 1 plane  -> FC 361->256 + ReLU -> FC 256->1 -> tanh
+// One workgroup of 256 threads per position; FC rows are read by whole
+// wavefronts (coalesced) and reduced with a butterfly.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+
+__global__ __launch_bounds__(256) void heads_k(const float* __restrict__ pol,
+                                               const float* __restrict__ val, HeadParams hp,
+                                               float temperature, float* __restrict__ policy,
+                                               float* __restrict__ logits,
+                                               float* __restrict__ value) {
+    __shared__ float xin[2 * kPts];
+    __shared__ float lg[362];
+    __shared__ float h1[256];
+    __shared__ float red[8];
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // ---- policy
+    for (int i = tid; i < 2 * kPts; i += 256) {
+        const int pl = i / kPts;
+        xin[i] = fmaxf(0.0f, hp.bn_pol_scale[pl] * (pol[(size_t)b * 2 * kPts + i] -
+                                                    hp.bn_pol_mean[pl]));
+    }
+    __syncthreads();
+    for (int o = wave; o < 362; o += 4) {
+        const float* w = hp.ip_pol_w + (size_t)o * (2 * kPts);
+        float s = 0.0f;
+        for (int i = lane; i < 2 * kPts; i += 64) s += w[i] * xin[i];
+        s = wave_sum(s);
+        if (lane == 0) lg[o] = hp.ip_pol_b[o] + s;
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int i = tid; i < 362; i += 256) m = fmaxf(m, lg[i]);
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float e[2];
+    float s = 0.0f;
+    for (int i = tid, q = 0; i < 362; i += 256, q++) {
+        e[q] = expf((lg[i] - m) / temperature);
+        s += e[q];
+    }
+    s = wave_sum(s);
+    if (lane == 0) red[4 + wave] = s;
+    __syncthreads();
+    const float denom = (red[4] + red[5]) + (red[6] + red[7]);
+    for (int i = tid, q = 0; i < 362; i += 256, q++) {
+        policy[(size_t)b * 362 + i] = e[q] / denom;
+        if (logits != nullptr) logits[(size_t)b * 362 + i] = lg[i];
+    }
+    __syncthreads();
+
+    // ---- value
+    for (int i = tid; i < kPts; i += 256)
+        xin[i] = fmaxf(0.0f, hp.bn_val_scale[0] * (val[(size_t)b * kPts + i] -
+                                                   hp.bn_val_mean[0]));
+    __syncthreads();
+    for (int o = wave; o < 256; o += 4) {
+        const float* w = hp.ip1_val_w + (size_t)o * kPts;
+        float acc = 0.0f;
+        for (int i = lane; i < kPts; i += 64) acc += w[i] * xin[i];
+        acc = wave_sum(acc);
+        if (lane == 0) h1[o] = fmaxf(0.0f, hp.ip1_val_b[o] + acc);
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float acc = 0.0f;
+        for (int i = lane; i < 256; i += 64) acc += hp.ip2_val_w[i] * h1[i];
+        acc = wave_sum(acc);
+        if (lane == 0) value[b] = tanhf(hp.ip2_val_b[0] + acc);
+    }
+}
+
+void launch_heads(const float* pol, const float* val, HeadParams hp, float temperature,
+                  float* policy, float* logits, float* value, int n, hipStream_t s) {
+    hipLaunchKernelGGL(heads_k, dim3(n), dim3(256), 0, s, pol, val, hp, temperature, policy,
+                       logits, value);
+}
+
+// ---------------------------------------------------------------------------
+#define INSTANTIATE(P)                                                                         \
+    template void launch_pack_input<P>(const float*, P*, int, int, int, hipStream_t,           \
+                                       LaunchTimer*);                                          \
+    template void launch_in_transform<P>(const P*, P*, int, int, int, hipStream_t,             \
+                                         LaunchTimer*);                                        \
+    template void launch_gemm<P>(const P*, const P*, P*, int, int, int, int, hipStream_t,      \
+                                 LaunchTimer*);                                                \
+    template void launch_out_transform<P>(const P*, const P*, P*, const float*, const float*,  \
+                                          float, int, int, int, hipStream_t, LaunchTimer*);    \
+    template void launch_head_conv<P>(const P*, const float*, float, float*, float*, int, int, \
+                                      hipStream_t, LaunchTimer*);                              \
+    template void launch_absmax<P>(const P*, size_t, float*, hipStream_t);
+INSTANTIATE(float)
+INSTANTIATE(half_t)
+
+}  // namespace lzhip

@@ -1,0 +1,77 @@
+"""CPU-side checks of the C-ABI library: it loads without a GPU, exports every
+symbol the header declares, and its host-only entry points agree with the oracle."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    header = open(os.path.join(ROOT, "include", "lzhip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(lzhip_[a-z0-9_]+)\s*\(", header)))
+    assert len(declared) >= 20
+    L = ctypes.CDLL(pkg.LIB_PATH)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert sorted(pkg.EXPORTS) == declared
+
+
+def test_version_and_error_string(pkg):
+    assert "gfx950" in pkg.version()
+    assert isinstance(pkg.lib().lzhip_last_error(), bytes)
+
+
+def test_null_arguments_are_rejected(pkg):
+    L = pkg.lib()
+    assert L.lzhip_create(64, 0, 1, 0, None) == pkg.EINVAL
+    assert L.lzhip_forward(None, None, None, None) == pkg.EINVAL
+    assert L.lzhip_drain(None) == pkg.EINVAL
+    assert L.lzhip_destroy(None) == pkg.OK
+    assert L.lzhip_winograd_transform_f(None, 1, 1, None) == pkg.EINVAL
+
+
+def test_transform_f_matches_oracle(pkg, orc):
+    rng = np.random.default_rng(0)
+    for K, C in ((8, 18), (5, 3), (16, 16)):
+        f = rng.standard_normal((K, C, 3, 3)).astype(np.float32)
+        got = pkg.winograd_transform_f(f, K, C)
+        want = orc.winograd_transform_f(f, K, C)
+        assert got.shape == want.shape == (36, C, K)
+        assert np.abs(got - want).max() <= 1e-6
+
+
+def test_bn_var_matches_oracle(pkg, orc):
+    v = np.random.default_rng(1).uniform(0.01, 4, 33).astype(np.float32)
+    assert np.abs(pkg.process_bn_var(v) - orc.process_bn_var(v)).max() <= 1e-7
+
+
+def test_python_pipe_validates_call_order(pkg, netgen):
+    pipe = pkg.HIPScheduler(pkg.FP32, 2)
+    with pytest.raises(ValueError):
+        pipe.forward(np.zeros(pkg.INPUT_SIZE, np.float32))
+    with pytest.raises(ValueError):
+        pipe.drain()
+
+
+def test_weights_file_round_trip(netgen, tmp_path):
+    net = netgen.make_network(1, 8, seed=5)
+    for name in ("w.txt", "w.txt.gz"):
+        p = tmp_path / name
+        netgen.save_weights(net, p)
+        back = netgen.load_weights(p)
+        assert (back.blocks, back.filters) == (1, 8)
+        for a, b in zip(net.lines(), back.lines()):
+            assert np.array_equal(np.asarray(a, np.float32).ravel(), np.asarray(b).ravel())
+    bad = tmp_path / "bad.txt"
+    bad.write_text("3\n")
+    with pytest.raises(ValueError):
+        netgen.load_weights(bad)
+    lines = open(tmp_path / "w.txt").read().split("\n")
+    (tmp_path / "short.txt").write_text("\n".join(lines[:-3]) + "\n")
+    with pytest.raises(ValueError):
+        netgen.load_weights(tmp_path / "short.txt")

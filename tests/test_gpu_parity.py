@@ -1,0 +1,220 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle on identical
+seeded networks and inputs.  Tolerances:
+  fp32: policy probabilities and value within 1e-4 max abs; raw planes rel-L2 <= 1e-5
+  fp16: policy within 2e-2, value within 2e-2; raw planes rel-L2 <= 2e-2
+Deep random-init networks saturate softmax/tanh, so the raw 1x1 planes and the
+logits are compared relatively as well.
+"""
+import threading
+
+import numpy as np
+import pytest
+
+from helpers import max_abs, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def make_pipes(pkg, netgen, orc, blocks, filters, seed, precision, max_batch):
+    net = netgen.make_network(blocks, filters, seed)
+    w, h = netgen.prepare(net)
+    w_ref, h_ref = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    ref = orc.OraclePipe()
+    ref.initialize(filters)
+    ref.push_weights(6, 18, filters, w_ref)
+    pipe = pkg.HIPScheduler(precision, max_batch)
+    pipe.initialize(filters)
+    pipe.push_weights(6, 18, filters, w)
+    pipe.push_heads(h)
+    return net, pipe, ref, h_ref
+
+
+@pytest.mark.parametrize("precision", [0, 1])
+@pytest.mark.parametrize("filters", [8, 64, 192])
+def test_single_layer_stages(pkg, netgen, orc, precision, filters):
+    """V, M and Y of one convolution layer against the oracle's stages, for the input
+    layer (18 planes) and a residual-tower layer with a skip connection."""
+    print("case: single_layer precision=%d filters=%d" % (precision, filters), flush=True)
+    net, pipe, ref, _ = make_pipes(pkg, netgen, orc, 1, filters, 40 + filters, precision, 4)
+    rng = np.random.default_rng(filters)
+    n = 3
+    tol = 1e-5 if precision == 0 else 4e-3
+    # layer 0 on real input planes
+    x = netgen.synthetic_inputs(n, seed=3)
+    V, M, Y = pipe.debug_layer(0, x)
+    for i in range(n):
+        Vr = orc.transform_in(x[i], 18)
+        Mr = orc.sgemm(ref.U[0], Vr, 18, filters)
+        Yr = orc.batchnorm(orc.transform_out(Mr, filters), ref.mean[0], ref.scale[0])
+        assert rel_l2(V[i], Vr) <= tol, "V layer0"
+        assert rel_l2(M[i], Mr) <= tol, "M layer0"
+        assert rel_l2(Y[i], Yr) <= tol, "Y layer0"
+    # layer 2 (second conv of the block) with a residual input
+    a = np.abs(rng.standard_normal((n, filters, 361))).astype(np.float32)
+    r = np.abs(rng.standard_normal((n, filters, 361))).astype(np.float32)
+    if precision == 1:  # make the inputs exactly representable in half precision
+        a = a.astype(np.float16).astype(np.float32)
+        r = r.astype(np.float16).astype(np.float32)
+    V, M, Y = pipe.debug_layer(2, a, r)
+    for i in range(n):
+        Vr = orc.transform_in(a[i], filters)
+        Mr = orc.sgemm(ref.U[2], Vr, filters, filters)
+        Yr = orc.batchnorm(orc.transform_out(Mr, filters), ref.mean[2], ref.scale[2], r[i])
+        assert rel_l2(V[i], Vr) <= tol, "V layer2"
+        assert rel_l2(M[i], Mr) <= tol, "M layer2"
+        assert rel_l2(Y[i], Yr) <= 2 * tol, "Y layer2"
+    pipe.close()
+
+
+def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None):
+    """Raw planes, logits, policy and value of the HIP pipe against the oracle."""
+    raw_tol = 1e-5 if precision == 0 else 2e-2
+    p_tol = 1e-4 if precision == 0 else 2e-2
+    policy, value, logits, pol, val = pipe.evaluate_batch(x, want_raw=True)
+    worst = dict(pol=0.0, val=0.0, policy=0.0, value=0.0)
+    for i in (range(x.shape[0]) if idx is None else idx):
+        rp, rv = ref.forward(x[i])
+        hd = orc.heads(h_ref, rp, rv)
+        worst["pol"] = max(worst["pol"], rel_l2(pol[i], rp))
+        worst["val"] = max(worst["val"], rel_l2(val[i], rv))
+        worst["policy"] = max(worst["policy"], max_abs(policy[i], hd["policy"]))
+        worst["value"] = max(worst["value"], abs(float(value[i]) - hd["value"]))
+        assert abs(float(policy[i].sum()) - 1.0) < 1e-4
+    print("parity", worst, flush=True)
+    assert worst["pol"] <= raw_tol and worst["val"] <= raw_tol, worst
+    assert worst["policy"] <= p_tol and worst["value"] <= p_tol, worst
+    return worst
+
+
+@pytest.mark.parametrize("blocks,filters,batch,precision", [
+    (1, 8, 3, 0),       # the shape of the reference's test network (1 block x 8 filters)
+    (6, 128, 1, 0),     # config 0: 6x128 fp32 batch 1
+    (15, 192, 8, 0),    # config 1: 15x192 fp32 batch 8
+    (1, 8, 3, 1),
+    (6, 128, 4, 1),     # config-0-sized net in fp16: the non-saturated fp16 check
+    (2, 96, 5, 1),
+])
+def test_forward_parity(pkg, netgen, orc, blocks, filters, batch, precision):
+    print("case: forward %dx%d b%d precision=%d" % (blocks, filters, batch, precision), flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, blocks, filters, 1000 + blocks, precision,
+                                       batch)
+    x = netgen.synthetic_inputs(batch, seed=blocks * 7 + filters)
+    check_outputs(pkg, orc, pipe, ref, h_ref, x, precision)
+    pipe.close()
+
+
+@pytest.mark.parametrize("blocks,filters,batch", [(20, 256, 32), (40, 256, 64)])
+def test_forward_parity_deep_fp16(pkg, netgen, orc, blocks, filters, batch):
+    """Configs 2 and 3 at full size; the oracle checks three positions of the batch."""
+    print("case: deep fp16 %dx%d b%d" % (blocks, filters, batch), flush=True)
+    orc.use_openblas()
+    try:
+        net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, blocks, filters, 2000 + blocks,
+                                           pkg.FP16, batch)
+        x = netgen.synthetic_inputs(batch, seed=blocks)
+        s = pipe.act_scales()
+        print("act scales: first %s last %s" % (s[:3], s[-3:]), flush=True)
+        assert np.all(s >= 1.0) and np.all(np.log2(s) == np.round(np.log2(s)))
+        check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16, idx=[0, batch // 2, batch - 1])
+        pipe.close()
+    finally:
+        orc.use_builtin()
+
+
+def test_golden_fixtures_on_device(pkg, netgen):
+    import os
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "tower_golden.npz"))
+    for tag in ("b1f8", "b2f16"):
+        blocks, filters, seed = [int(v) for v in g[tag + "_cfg"]]
+        net = netgen.make_network(blocks, filters, seed)
+        w, h = netgen.prepare(net)
+        for precision, raw_tol, p_tol in ((pkg.FP32, 1e-5, 1e-4), (pkg.FP16, 2e-2, 2e-2)):
+            pipe = pkg.HIPScheduler(precision, 4)
+            pipe.initialize(filters)
+            pipe.push_weights(6, 18, filters, w)
+            pipe.push_heads(h)
+            policy, value, logits, pol, val = pipe.evaluate_batch(g[tag + "_x"], want_raw=True)
+            assert rel_l2(pol, g[tag + "_pol"]) <= raw_tol
+            assert rel_l2(val, g[tag + "_val"]) <= raw_tol
+            assert max_abs(policy, g[tag + "_policy"]) <= p_tol
+            assert max_abs(value, g[tag + "_value"]) <= p_tol
+            pipe.close()
+
+
+@pytest.mark.parametrize("precision", [0, 1])
+def test_batch_composition_does_not_change_results(pkg, netgen, orc, precision):
+    """A position evaluated alone, in a partial batch and in a full batch gives
+    bit-identical planes (rows of the GEMM are independent)."""
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 2, 64, 77, precision, 8)
+    x = netgen.synthetic_inputs(8, seed=5)
+    pol8, val8 = pipe.forward_batch(x)
+    pol3, val3 = pipe.forward_batch(x[2:5])
+    pol1, val1 = pipe.forward_batch(x[4:5])
+    assert np.array_equal(pol8[2:5], pol3) and np.array_equal(val8[2:5], val3)
+    assert np.array_equal(pol8[4:5], pol1) and np.array_equal(val8[4:5], val1)
+    # a larger batch after a smaller one (stale rows in the padded tile range)
+    pol8b, val8b = pipe.forward_batch(x)
+    assert np.array_equal(pol8, pol8b) and np.array_equal(val8, val8b)
+    with pytest.raises(ValueError):
+        pipe.forward_batch(np.zeros((9, 18, 361), np.float32))
+    pipe.close()
+
+
+def test_scheduler_concurrent_requests(pkg, netgen, orc):
+    """Many threads call forward() at once: each gets its own position's result,
+    identical to the batch executor's, and the batches fill."""
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 2, 64, 78, pkg.FP32, 8)
+    x = netgen.synthetic_inputs(24, seed=6)
+    pol_ref = np.concatenate([pipe.forward_batch(x[i:i + 8])[0] for i in range(0, 24, 8)])
+    out = [None] * 24
+    pipe.reset_stats()
+
+    def work(i):
+        for rep in range(3):
+            out[i] = pipe.forward(x[i])
+
+    th = [threading.Thread(target=work, args=(i,)) for i in range(24)]
+    [t.start() for t in th]
+    [t.join() for t in th]
+    for i in range(24):
+        assert np.array_equal(out[i][0], pol_ref[i])
+    st = pipe.stats()
+    assert st["requests"] == 72 and st["halted"] == 0
+    assert st["max_batch_seen"] <= 8 and st["batches"] < 72
+    pipe.close()
+
+
+def test_drain_and_resume(pkg, netgen, orc):
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, 8, 79, pkg.FP32, 4)
+    x = netgen.synthetic_inputs(1, seed=7)[0]
+    pipe.forward(x)
+    pipe.drain()
+    with pytest.raises(pkg.NetworkHaltException):
+        pipe.forward(x)
+    pipe.resume()
+    pol, val = pipe.forward(x)
+    rp, rv = ref.forward(x)
+    assert rel_l2(pol, rp) < 1e-5
+    assert pipe.stats()["halted"] == 1
+    pipe.close()
+
+
+def test_device_resident_forward_and_profile(pkg, netgen, orc):
+    """The device-pointer entry point (what the bench times) gives the same planes as
+    the host entry point, and the per-kernel timing hook reports every launch."""
+    import torch
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 2, 64, 80, pkg.FP16, 4)
+    x = netgen.synthetic_inputs(4, seed=8)
+    pol_h, val_h = pipe.forward_batch(x)
+    d_in = torch.from_numpy(x).cuda()
+    d_pol = torch.zeros(4, 722, device="cuda")
+    d_val = torch.zeros(4, 361, device="cuda")
+    torch.cuda.synchronize()
+    pipe.forward_batch_device(4, d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
+    pipe.sync()
+    assert np.array_equal(d_pol.cpu().numpy(), pol_h) and np.array_equal(d_val.cpu().numpy(), val_h)
+    ms, cnt = pipe.profile_forward(4, d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
+    assert list(cnt) == [1, 5, 5, 5, 1]
+    assert np.all(ms > 0) and np.all(ms < 50)
+    assert np.array_equal(d_pol.cpu().numpy(), pol_h)
+    pipe.close()

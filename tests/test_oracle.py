@@ -1,0 +1,214 @@
+"""Pins the CPU oracle (oracle/lz_oracle.c) before anything is compared with it.
+
+The reference holds no numeric vectors for this path, and its CPU pipe cannot
+be compiled in this image, so every oracle function is pinned by what the
+mathematics fixes: literal transform matrices applied densely in float64,
+direct zero-padded 3x3 correlation, and textbook closed forms -- chosen so
+that a transposed operand, a wrong index or a dropped term fails.
+"""
+import numpy as np
+import pytest
+
+from helpers import conv3x3_f64, heads_f64, max_abs, rel_l2, tower_f64
+
+S2 = np.sqrt(2.0)
+# The literal matrices (reference src/Network.cpp:166-172, src/CPUPipe.cpp:81-87, :220-224).
+G = np.array([[1, 0, 0], [-2 / 3, -S2 / 3, -1 / 3], [-2 / 3, S2 / 3, -1 / 3],
+              [1 / 6, S2 / 6, 1 / 3], [1 / 6, -S2 / 6, 1 / 3], [0, 0, 1]])
+BT = np.array([[1, 0, -5 / 2, 0, 1, 0], [0, -S2, -2, S2 / 2, 1, 0], [0, S2, -2, -S2 / 2, 1, 0],
+               [0, -S2 / 2, -1 / 2, S2, 1, 0], [0, S2 / 2, -1 / 2, -S2, 1, 0],
+               [0, 1, 0, -5 / 2, 0, 1]])
+AT = np.array([[1, 1, 1, 1, 1, 0], [0, S2 / 2, -S2 / 2, S2, -S2, 0], [0, 1 / 2, 1 / 2, 2, 2, 0],
+               [0, S2 / 4, -S2 / 4, 2 * S2, -2 * S2, 1]])
+
+
+def test_matrices_are_a_winograd_triple():
+    """A^T[(G g G^T) * (B^T d B)]A == valid correlation of a 6x6 patch with a 3x3 filter.
+    Guards the test's own literal matrices."""
+    rng = np.random.default_rng(1)
+    g, d = rng.standard_normal((3, 3)), rng.standard_normal((6, 6))
+    y = AT @ ((G @ g @ G.T) * (BT @ d @ BT.T)) @ AT.T
+    want = np.array([[np.sum(d[i:i + 3, j:j + 3] * g) for j in range(4)] for i in range(4)])
+    assert np.abs(y - want).max() < 1e-12
+
+
+def test_transform_f_layout_and_values(orc):
+    rng = np.random.default_rng(2)
+    K, C = 5, 3  # distinct, so a swapped index shows
+    f = rng.standard_normal((K, C, 3, 3)).astype(np.float32)
+    U = orc.winograd_transform_f(f, K, C)
+    assert U.shape == (36, C, K)
+    want = np.einsum("xi,ocij,nj->xnco", G, f.astype(np.float64), G).reshape(36, C, K)
+    assert max_abs(U, want) < 2e-6
+    # outputs divisible by 8 takes the reference's buffered branch (src/Network.cpp:176-181)
+    f8 = rng.standard_normal((16, 2, 3, 3)).astype(np.float32)
+    want8 = np.einsum("xi,ocij,nj->xnco", G, f8.astype(np.float64), G).reshape(36, 2, 16)
+    assert max_abs(orc.winograd_transform_f(f8, 16, 2), want8) < 2e-6
+
+
+def _patches(x):
+    """x [C][19][19] -> [C][25][6][6] zero-haloed patches, tile = by*5+bx."""
+    C = x.shape[0]
+    pad = np.zeros((C, 24, 24))
+    pad[:, 1:20, 1:20] = x
+    out = np.empty((C, 25, 6, 6))
+    for by in range(5):
+        for bx in range(5):
+            out[:, by * 5 + bx] = pad[:, 4 * by:4 * by + 6, 4 * bx:4 * bx + 6]
+    return out
+
+
+def test_transform_in_layout_and_values(orc):
+    rng = np.random.default_rng(3)
+    C = 4
+    x = rng.standard_normal((C, 19, 19)).astype(np.float32)
+    V = orc.transform_in(x, C)
+    d = _patches(x.astype(np.float64))
+    want = np.einsum("xi,cpij,nj->xncp", BT, d, BT).reshape(36, C, 25)
+    assert V.shape == (36, C, 25)
+    assert max_abs(V, want) < 1e-4 * np.abs(want).max()
+
+
+def test_sgemm_contracts_over_input_channels(orc):
+    rng = np.random.default_rng(4)
+    C, K = 6, 9
+    U = rng.standard_normal((36, C, K)).astype(np.float32)
+    V = rng.standard_normal((36, C, 25)).astype(np.float32)
+    want = np.einsum("bck,bcp->bkp", U.astype(np.float64), V.astype(np.float64))
+    orc.use_builtin()
+    assert max_abs(orc.sgemm(U, V, C, K), want) < 1e-5
+    if orc.use_openblas() != "builtin":
+        assert max_abs(orc.sgemm(U, V, C, K), want) < 1e-5
+    orc.use_builtin()
+
+
+def test_transform_out_layout_clipping(orc):
+    rng = np.random.default_rng(5)
+    K = 3
+    M = rng.standard_normal((36, K, 25)).astype(np.float32)
+    Y = orc.transform_out(M, K).reshape(K, 19, 19)
+    m = M.astype(np.float64).reshape(6, 6, K, 25)
+    tiles = np.einsum("ix,xnkp,jn->kpij", AT, m, AT)
+    want = np.zeros((K, 20, 20))
+    for by in range(5):
+        for bx in range(5):
+            want[:, 4 * by:4 * by + 4, 4 * bx:4 * bx + 4] = tiles[:, by * 5 + bx]
+    assert max_abs(Y, want[:, :19, :19]) < 1e-4
+
+
+@pytest.mark.parametrize("C,K", [(18, 8), (7, 5), (32, 16)])
+def test_winograd_chain_equals_direct_convolution(orc, C, K):
+    rng = np.random.default_rng(6)
+    f = (rng.standard_normal((K, C, 3, 3)) / np.sqrt(9 * C)).astype(np.float32)
+    x = rng.standard_normal((C, 19, 19)).astype(np.float32)
+    U = orc.winograd_transform_f(f, K, C)
+    Y = orc.transform_out(orc.sgemm(U, orc.transform_in(x, C), C, K), K)
+    want = conv3x3_f64(x[None], f)[0].reshape(K, 361)
+    assert rel_l2(Y, want) < 2e-6
+    # corners and edges see the zero halo and the 19x19 clipping
+    Yb, wb = Y.reshape(K, 19, 19), want.reshape(K, 19, 19)
+    for sl in [(0, 0), (0, 18), (18, 0), (18, 18), (9, 18), (18, 9)]:
+        assert np.abs(Yb[:, sl[0], sl[1]] - wb[:, sl[0], sl[1]]).max() < 1e-4
+
+
+def test_bn_var_and_batchnorm(orc):
+    rng = np.random.default_rng(7)
+    var = rng.uniform(0.1, 3, 6).astype(np.float32)
+    assert max_abs(orc.process_bn_var(var), 1 / np.sqrt(var.astype(np.float64) + 1e-5)) < 1e-6
+    x = rng.standard_normal((6, 361)).astype(np.float32)
+    mean = rng.standard_normal(6).astype(np.float32)
+    s = rng.uniform(0.5, 2, 6).astype(np.float32)
+    res = rng.standard_normal((6, 361)).astype(np.float32)
+    want = np.maximum(0, s[:, None] * (x - mean[:, None]))
+    assert max_abs(orc.batchnorm(x, mean, s), want) < 1e-6
+    want_r = np.maximum(0, s[:, None] * (x - mean[:, None]) + res)
+    assert max_abs(orc.batchnorm(x, mean, s, res), want_r) < 1e-6
+    assert (orc.batchnorm(x, mean, s) >= 0).all()
+
+
+def test_convolve1(orc):
+    rng = np.random.default_rng(8)
+    C = 11
+    x = rng.standard_normal((C, 361)).astype(np.float32)
+    w = rng.standard_normal((2, C)).astype(np.float32)
+    assert max_abs(orc.convolve1(x, w, 2, C), w.astype(np.float64) @ x.astype(np.float64)) < 1e-5
+
+
+@pytest.mark.parametrize("blocks,filters", [(1, 8), (2, 16)])
+def test_forward_wiring_against_float64_direct_model(orc, netgen, blocks, filters):
+    """Layer order, residual wiring (skip = block input after its ReLU, added before
+    the last ReLU), bias folding and the head convolutions."""
+    net = netgen.make_network(blocks, filters, seed=11)
+    # non-zero conv biases exercise the folding into the BN means
+    rng = np.random.default_rng(12)
+    for l in range(net.n_layers):
+        net.conv_b[l] = (rng.standard_normal(filters) * 0.05).astype(np.float32)
+    x = netgen.synthetic_inputs(2, seed=13)
+    w, _ = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    pipe = orc.OraclePipe()
+    pipe.initialize(filters)
+    pipe.push_weights(6, 18, filters, w)
+    want = tower_f64(net, x)
+    for i in range(2):
+        pol, val, trace = pipe.forward(x[i], trace=True)
+        for l in range(net.n_layers):
+            assert rel_l2(trace[l], want["acts"][l][i].reshape(filters, 361)) < 1e-5, l
+        assert rel_l2(pol, want["pol"][i]) < 1e-5
+        assert rel_l2(val, want["val"][i]) < 1e-5
+
+
+def test_heads_against_float64(orc, netgen):
+    net = netgen.make_network(1, 8, seed=21)
+    rng = np.random.default_rng(22)
+    net.pol_fc_b = (rng.standard_normal(362) * 0.1).astype(np.float32)
+    net.val_fc1_b = (rng.standard_normal(256) * 0.1).astype(np.float32)
+    net.val_fc2_b = (rng.standard_normal(1) * 0.1).astype(np.float32)
+    net.pol_conv_b = (rng.standard_normal(2) * 0.1).astype(np.float32)
+    _, h = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    pol = rng.standard_normal(722).astype(np.float32)
+    val = rng.standard_normal(361).astype(np.float32)
+    for temp in (1.0, 0.7):
+        got = orc.heads(h, pol, val, temp)
+        want = heads_f64(net, pol, val, temp)
+        assert max_abs(got["logits"], want["logits"]) < 1e-5
+        assert max_abs(got["policy"], want["policy"]) < 1e-6
+        assert abs(got["policy"].sum() - 1) < 1e-5
+        assert abs(got["value"] - want["value"]) < 1e-6
+        assert abs(got["winrate"] - want["winrate"]) < 1e-6
+
+
+def test_threaded_forward_matches_single(orc, netgen):
+    net = netgen.make_network(1, 8, seed=31)
+    x = netgen.synthetic_inputs(5, seed=32)
+    w, _ = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    pipe = orc.OraclePipe()
+    pipe.initialize(8)
+    pipe.push_weights(6, 18, 8, w)
+    pol, val, secs = pipe.forward_many(x, threads=3)
+    assert secs > 0
+    for i in range(5):
+        p, v = pipe.forward(x[i])
+        assert np.array_equal(p, pol[i]) and np.array_equal(v, val[i])
+
+
+def test_golden_fixtures(orc, netgen):
+    """The committed fixtures (tests/golden/make_golden.py: float64 direct-convolution
+    model) agree with the oracle."""
+    import os
+    path = os.path.join(os.path.dirname(__file__), "golden", "tower_golden.npz")
+    g = np.load(path)
+    for tag in ("b1f8", "b2f16"):
+        blocks, filters, seed = [int(v) for v in g[tag + "_cfg"]]
+        net = netgen.make_network(blocks, filters, seed)
+        x = g[tag + "_x"]
+        w, h = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+        pipe = orc.OraclePipe()
+        pipe.initialize(filters)
+        pipe.push_weights(6, 18, filters, w)
+        for i in range(x.shape[0]):
+            pol, val = pipe.forward(x[i])
+            assert rel_l2(pol, g[tag + "_pol"][i]) < 1e-5
+            assert rel_l2(val, g[tag + "_val"][i]) < 1e-5
+            hd = orc.heads(h, pol, val)
+            assert max_abs(hd["policy"], g[tag + "_policy"][i]) < 1e-5
+            assert abs(hd["value"] - g[tag + "_value"][i]) < 1e-5
