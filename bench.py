@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Headline benchmark: NN evaluations per second of the 40-block x 256-filter
+network, fp16 storage / fp32 accumulate, batch 64, on one MI355X.
+
+A step is one forward pass (residual tower + 1x1 heads) over one batch of 64
+synthetic positions that already sit in device memory.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+PEAK_MFMA_F16 = 2.5e15   # dense fp16 matrix FLOP/s, MI355X
+PEAK_MFMA_F32 = 157.3e12
+PEAK_HBM = 8.0e12        # bytes/s
+
+
+def gemm_flops(batch, filters, n_layers):
+    """Algorithmic flops of the 36 batched GEMMs of one forward:
+    2 * 36 * (25*batch) * F * (18 + (L-1)*F)."""
+    return 2.0 * 36 * 25 * batch * filters * (18 + (n_layers - 1) * filters)
+
+
+def transform_bytes(batch, filters, n_layers, e):
+    """Algorithmic HBM bytes of the input and output transforms of one forward
+    (unfused minimal traffic: activations in + Winograd tiles out, and back)."""
+    T = 25 * batch
+    act = batch * filters * 361 * e
+    tiles = 36 * filters * T * e
+    in_t = (batch * 18 * 361 * e + 36 * 18 * T * e) + (n_layers - 1) * (act + tiles)
+    n_res = (n_layers - 1) // 2
+    out_t = n_layers * (tiles + act + 2 * filters * 4) + n_res * act
+    return in_t, out_t
+
+
+def cpu_baseline(orc, netgen, net, x, seconds_budget=20.0):
+    """CPU oracle timed on this host: independent single-position forwards on all
+    the cores this process may use (the shape of the reference's netbench)."""
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = max(1, min(16, cores))
+    provider = orc.use_openblas()
+    w_ref, _ = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    ref = orc.OraclePipe()
+    ref.initialize(net.filters)
+    ref.push_weights(6, 18, net.filters, w_ref)
+    t0 = time.perf_counter()
+    ref.forward(x[0])
+    one = time.perf_counter() - t0
+    per_thread = max(1, int(seconds_budget / max(one, 1e-3)))
+    per_thread = min(per_thread, 8)
+    n = cores * per_thread
+    xs = np.concatenate([x] * (n // x.shape[0] + 1))[:n]
+    pol, val, secs = ref.forward_many(xs, threads=cores)
+    return {
+        "value": n / secs, "unit": "evals/s", "cores": cores, "kind": "port",
+        "sample": "%d single-position forwards of the same %dx%d net (CPU oracle, fp32, "
+                  "Winograd F(4x4,3x3), sgemm=%s, 1 BLAS thread per call) on %d threads, %.1f s"
+                  % (n, net.blocks, net.filters, provider, cores, secs),
+    }, (pol, val)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--blocks", type=int, default=40)
+    ap.add_argument("--filters", type=int, default=256)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--precision", choices=["fp16", "fp32"], default="fp16")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-reps", type=int, default=5)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (one replica per GPU, no "
+              "collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    pkg = entry.load_package()
+    import leela_zero_amd.netgen as netgen
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+
+    B, F, blocks = args.batch, args.filters, args.blocks
+    prec = pkg.FP16 if args.precision == "fp16" else pkg.FP32
+    net = netgen.make_network(blocks, F, seed=2025)
+    x = netgen.synthetic_inputs(B, seed=2026)
+    w, h = netgen.prepare(net)
+    pipe = pkg.HIPScheduler(prec, B, device=0)
+    pipe.initialize(F)
+    pipe.push_weights(6, 18, F, w)
+    nl = net.n_layers
+
+    d_in = torch.from_numpy(x).cuda()
+    d_pol = torch.zeros(B, 722, device="cuda")
+    d_val = torch.zeros(B, 361, device="cuda")
+    torch.cuda.synchronize()
+    ptrs = (d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
+
+    for _ in range(args.warmup):
+        pipe.forward_batch_device(B, *ptrs)
+    pipe.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        pipe.forward_batch_device(B, *ptrs)
+    pipe.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    evals = B * args.steps / dt
+
+    # per-kernel-class device time, measured live with HIP events on the pipe's stream
+    ms = np.zeros(pkg.K_COUNT)
+    cnt = np.zeros(pkg.K_COUNT)
+    for _ in range(args.profile_reps):
+        m, c = pipe.profile_forward(B, *ptrs)
+        ms += m
+        cnt += c
+    ms /= args.profile_reps
+    cnt /= args.profile_reps
+    e = 2 if prec == pkg.FP16 else 4
+    gf = gemm_flops(B, F, nl)
+    in_b, out_b = transform_bytes(B, F, nl, e)
+    peak = PEAK_MFMA_F16 if prec == pkg.FP16 else PEAK_MFMA_F32
+    gemm_rate = gf / (ms[pkg.K_GEMM] * 1e-3)
+    roofline = {
+        "kernel": "wino_gemm_k (36-way batched Winograd GEMM)",
+        "bound": "mfma", "achieved": gemm_rate / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
+        "frac": gemm_rate / peak, "traffic": None,
+        "avg_launch_us": ms[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],
+        "launches_per_forward": int(cnt[pkg.K_GEMM]),
+        "flops_per_launch": gf / cnt[pkg.K_GEMM],
+    }
+    in_rate = in_b / (ms[pkg.K_IN] * 1e-3)
+    out_rate = out_b / (ms[pkg.K_OUT] * 1e-3)
+    transforms = {
+        "in_transform": {"bound": "hbm", "achieved": in_rate / 1e9, "peak": PEAK_HBM / 1e9,
+                         "unit": "GB/s", "frac": in_rate / PEAK_HBM,
+                         "avg_launch_us": ms[pkg.K_IN] * 1e3 / cnt[pkg.K_IN]},
+        "out_transform": {"bound": "hbm", "achieved": out_rate / 1e9, "peak": PEAK_HBM / 1e9,
+                          "unit": "GB/s", "frac": out_rate / PEAK_HBM,
+                          "avg_launch_us": ms[pkg.K_OUT] * 1e3 / cnt[pkg.K_OUT]},
+    }
+    kernel_ms = {pkg.KERNEL_CLASSES[k]: float(ms[k]) for k in range(pkg.K_COUNT)}
+
+    # parity spot check + CPU baseline (oracle as checker / reported baseline only)
+    cpu = None
+    if not args.no_cpu_baseline:
+        orc = entry.load_oracle()
+        cpu, (rpol, rval) = cpu_baseline(orc, netgen, net, x)
+        pol = d_pol.cpu().numpy()
+        k = min(B, rpol.shape[0])
+        rel = float(np.linalg.norm(pol[:k] - rpol[:k]) / max(np.linalg.norm(rpol[:k]), 1e-30))
+        cpu["raw_policy_plane_rel_l2_vs_gpu"] = rel
+    pipe.close()
+
+    out = {
+        "metric": "NN evals/sec at 40x256 fp16 b64 on 1 MI355X; Winograd GEMM MFMA util %",
+        "value": evals, "unit": "evals/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 storage, f32 accumulate" if prec == pkg.FP16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": "%d blocks x %d filters, %s, batch %d (BASELINE configs[3] when "
+                               "40x256 fp16 b64), %d conv layers + 1x1 heads per step"
+                               % (blocks, F, args.precision, B, nl),
+                   "inputs": "device-resident fp32 NCHW [%d][18][361]" % B},
+        "roofline": roofline,
+        "roofline_transforms": transforms,
+        "kernel_ms_per_forward": kernel_ms,
+        "gemm_mfma_util_pct": 100.0 * gemm_rate / peak,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

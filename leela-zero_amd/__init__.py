@@ -68,6 +68,13 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise LzhipError("%s is missing: run __graft_entry__.build() (hipcc) first; "
                              "there is no fallback implementation" % LIB_PATH)
+        # A process that also uses torch-ROCm must hold ONE HIP runtime: torch ships its
+        # own copy, and whichever copy is loaded second finds no devices.  Loading
+        # torch first makes this library bind to torch's copy (same SONAME).
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         L.lzhip_last_error.restype = ctypes.c_char_p
         L.lzhip_version.restype = ctypes.c_char_p

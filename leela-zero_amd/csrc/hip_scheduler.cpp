@@ -182,8 +182,11 @@ void HIPScheduler::worker() {
             };
             if (m_queue.size() < want() && m_max_wait_us > 0) {
                 const size_t before = m_queue.size();
+                // system_clock: waits on it map to pthread_cond_timedwait, which thread
+                // sanitizers model; the grace period is far too short for clock steps
+                // to matter.
                 const auto deadline =
-                    std::chrono::steady_clock::now() + std::chrono::microseconds(m_wait_us);
+                    std::chrono::system_clock::now() + std::chrono::microseconds(m_wait_us);
                 m_cv.wait_until(lk, deadline, [&] {
                     return !m_running || m_queue.empty() || m_queue.size() >= want();
                 });

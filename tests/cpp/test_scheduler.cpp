@@ -1,0 +1,173 @@
+// Host-only test of the batching scheduler with a stand-in executor, meant to be
+// built with -fsanitize=thread.  Checks the invariants the reference's scheduler
+// promises its callers (reference src/OpenCLScheduler.cpp:256-441):
+//   * every request is answered exactly once, with its own position's data;
+//   * a batch never exceeds max_batch;
+//   * drain() releases every waiter with a halt, later calls halt at once,
+//     resume() needs an empty queue and re-opens the pipe;
+//   * destruction with idle and with blocked callers ends cleanly;
+//   * an executor failure reaches the caller as an exception.
+#include <atomic>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <stdexcept>
+#include <thread>
+#include <vector>
+
+#include "forward_pipe.h"
+
+using namespace lzhip;
+
+// The scheduler's translation unit refers to the device factory; no device here.
+namespace lzhip {
+std::unique_ptr<BatchExecutor> make_hip_pipe(int, int, int, int) {
+    throw std::runtime_error("no device in the scheduler test");
+}
+}  // namespace lzhip
+
+#define CHECK(cond)                                                        \
+    do {                                                                   \
+        if (!(cond)) {                                                     \
+            std::fprintf(stderr, "FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            std::exit(1);                                                  \
+        }                                                                  \
+    } while (0)
+
+// pol[i] = in[0] + i, val[i] = in[1] - i : each answer identifies its own request.
+class FakeExec : public BatchExecutor {
+public:
+    FakeExec(int mb, int delay_us) : m_mb(mb), m_delay(delay_us) {}
+    int max_batch() const override { return m_mb; }
+    void forward_batch(int n, const float* in, float* pol, float* val) override {
+        if (n < 1 || n > m_mb) { oversize = true; }
+        if (fail_next.exchange(false)) throw std::runtime_error("injected failure");
+        std::this_thread::sleep_for(std::chrono::microseconds(m_delay));
+        for (int b = 0; b < n; b++) {
+            const float* x = in + (size_t)b * LZHIP_INPUT_SIZE;
+            for (int i = 0; i < LZHIP_POL_SIZE; i++) pol[(size_t)b * LZHIP_POL_SIZE + i] = x[0] + i;
+            for (int i = 0; i < LZHIP_VAL_SIZE; i++) val[(size_t)b * LZHIP_VAL_SIZE + i] = x[1] - i;
+        }
+        calls++;
+        positions += n;
+    }
+    std::atomic<bool> oversize{false}, fail_next{false};
+    std::atomic<int> calls{0}, positions{0};
+private:
+    int m_mb, m_delay;
+};
+
+static void one_call(HIPScheduler& s, float a, float b, std::atomic<int>& ok,
+                     std::atomic<int>& halted) {
+    std::vector<float> in(LZHIP_INPUT_SIZE, 0.0f), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
+    in[0] = a;
+    in[1] = b;
+    try {
+        s.forward(in, pol, val);
+        for (int i = 0; i < LZHIP_POL_SIZE; i++) CHECK(pol[i] == a + i);
+        for (int i = 0; i < LZHIP_VAL_SIZE; i++) CHECK(val[i] == b - i);
+        ok++;
+    } catch (const NetworkHaltException&) {
+        halted++;
+    }
+}
+
+static void test_concurrent(int threads, int mb, int reps) {
+    auto* fe = new FakeExec(mb, 200);
+    HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
+    std::atomic<int> ok{0}, halted{0};
+    std::vector<std::thread> th;
+    for (int t = 0; t < threads; t++)
+        th.emplace_back([&, t] {
+            for (int r = 0; r < reps; r++) one_call(s, (float)(t * 1000 + r), (float)(r - t), ok, halted);
+        });
+    for (auto& t : th) t.join();
+    CHECK(ok == threads * reps && halted == 0);
+    CHECK(!fe->oversize);
+    CHECK(fe->positions == threads * reps);
+    const lzhip_stats st = s.stats();
+    CHECK(st.requests == (uint64_t)threads * reps);
+    CHECK(st.max_batch_seen <= (uint32_t)mb);
+    CHECK(st.batches == (uint64_t)fe->calls.load());
+    if (threads >= 2 * mb) CHECK(st.batches < (uint64_t)threads * reps);  // it did batch
+    std::printf("concurrent threads=%d mb=%d: %llu batches for %llu requests, max %u\n", threads,
+                mb, (unsigned long long)st.batches, (unsigned long long)st.requests,
+                st.max_batch_seen);
+}
+
+static void test_drain_resume() {
+    auto* fe = new FakeExec(4, 20000);  // slow executor: requests pile up in the queue
+    HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
+    s.set_max_wait_us(0);
+    std::atomic<int> ok{0}, halted{0};
+    std::vector<std::thread> th;
+    for (int t = 0; t < 16; t++) th.emplace_back([&, t] { one_call(s, (float)t, 1.0f, ok, halted); });
+    std::this_thread::sleep_for(std::chrono::milliseconds(5));
+    s.drain();
+    for (auto& t : th) t.join();
+    CHECK(ok + halted == 16);
+    CHECK(halted >= 1);  // the slow executor cannot have served all 16 in 5 ms
+    // while drained every new call halts immediately
+    one_call(s, 1.0f, 2.0f, ok, halted);
+    CHECK(ok + halted == 17);
+    const int halted_before = halted;
+    s.resume();
+    one_call(s, 3.0f, 4.0f, ok, halted);
+    CHECK(halted == halted_before);
+    CHECK(s.stats().halted == (uint64_t)halted_before);
+    std::printf("drain/resume: %d served, %d halted\n", ok.load(), halted.load());
+}
+
+static void test_destroy_with_waiters() {
+    std::atomic<int> ok{0}, halted{0};
+    std::vector<std::thread> th;
+    {
+        auto* fe = new FakeExec(2, 30000);
+        auto s = std::make_unique<HIPScheduler>(std::unique_ptr<BatchExecutor>(fe));
+        s->set_max_wait_us(0);
+        for (int t = 0; t < 8; t++) th.emplace_back([&, t, p = s.get()] { one_call(*p, (float)t, 0.0f, ok, halted); });
+        std::this_thread::sleep_for(std::chrono::milliseconds(5));
+        s->drain();  // callers must be out of forward() before the object may die
+        for (auto& t : th) t.join();
+    }
+    CHECK(ok + halted == 8);
+    { HIPScheduler idle{std::unique_ptr<BatchExecutor>(new FakeExec(2, 10))}; }
+    std::printf("destroy: %d served, %d halted\n", ok.load(), halted.load());
+}
+
+static void test_executor_failure() {
+    auto* fe = new FakeExec(4, 10);
+    HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
+    fe->fail_next = true;
+    std::vector<float> in(LZHIP_INPUT_SIZE, 0.0f), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
+    bool threw = false;
+    try {
+        s.forward(in, pol, val);
+    } catch (const std::runtime_error& e) {
+        threw = std::string(e.what()) == "injected failure";
+    }
+    CHECK(threw);
+    std::atomic<int> ok{0}, halted{0};
+    one_call(s, 5.0f, 6.0f, ok, halted);  // the pipe keeps working afterwards
+    CHECK(ok == 1);
+    bool bad = false;
+    try {
+        std::vector<float> small(3);
+        s.forward(small, pol, val);
+    } catch (const std::invalid_argument&) {
+        bad = true;
+    }
+    CHECK(bad);
+    std::printf("executor failure propagated\n");
+}
+
+int main() {
+    test_concurrent(1, 4, 20);
+    test_concurrent(16, 32, 30);   // fewer callers than max_batch: must still batch, never stall
+    test_concurrent(48, 8, 20);
+    test_drain_resume();
+    test_destroy_with_waiters();
+    test_executor_failure();
+    std::printf("scheduler tests passed\n");
+    return 0;
+}
