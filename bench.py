@@ -29,15 +29,22 @@ def gemm_flops(batch, filters, n_layers):
 
 
 def transform_bytes(batch, filters, n_layers, e):
-    """Algorithmic HBM bytes of the input and output transforms of one forward
-    (unfused minimal traffic: activations in + Winograd tiles out, and back)."""
+    """Algorithmic HBM bytes per forward of the three transform kernel classes:
+    external inputs + outputs of each launch, nothing counted twice.
+      in_transform   (layer 0 only): input planes packed to 64 channels + V_0
+      out_in         (layers 0..L-2): M_l in, V_{l+1} out, + the activation out on block
+                     ends (layer 0 and second convs) + the skip activation in (l >= 2)
+      out_transform  (last layer): M in, skip in, activation out"""
     T = 25 * batch
     act = batch * filters * 361 * e
     tiles = 36 * filters * T * e
-    in_t = (batch * 18 * 361 * e + 36 * 18 * T * e) + (n_layers - 1) * (act + tiles)
-    n_res = (n_layers - 1) // 2
-    out_t = n_layers * (tiles + act + 2 * filters * 4) + n_res * act
-    return in_t, out_t
+    bn = 2 * filters * 4
+    in_t = batch * 64 * 361 * e + 36 * 64 * T * e
+    n_fused = n_layers - 1
+    n_block_end = (n_layers - 1) // 2          # l = 0, 2, ..., L-3
+    fused = n_fused * (2 * tiles + bn) + n_block_end * act + max(0, n_block_end - 1) * act
+    out_t = tiles + act + bn + (act if n_layers >= 3 else 0)
+    return in_t, out_t, fused
 
 
 def cpu_baseline(orc, netgen, net, x, seconds_budget=20.0):
@@ -130,7 +137,7 @@ def main():
     cnt /= args.profile_reps
     e = 2 if prec == pkg.FP16 else 4
     gf = gemm_flops(B, F, nl)
-    in_b, out_b = transform_bytes(B, F, nl, e)
+    in_b, out_b, fused_b = transform_bytes(B, F, nl, e)
     peak = PEAK_MFMA_F16 if prec == pkg.FP16 else PEAK_MFMA_F32
     gemm_rate = gf / (ms[pkg.K_GEMM] * 1e-3)
     roofline = {
@@ -141,16 +148,18 @@ def main():
         "launches_per_forward": int(cnt[pkg.K_GEMM]),
         "flops_per_launch": gf / cnt[pkg.K_GEMM],
     }
-    in_rate = in_b / (ms[pkg.K_IN] * 1e-3)
-    out_rate = out_b / (ms[pkg.K_OUT] * 1e-3)
-    transforms = {
-        "in_transform": {"bound": "hbm", "achieved": in_rate / 1e9, "peak": PEAK_HBM / 1e9,
-                         "unit": "GB/s", "frac": in_rate / PEAK_HBM,
-                         "avg_launch_us": ms[pkg.K_IN] * 1e3 / cnt[pkg.K_IN]},
-        "out_transform": {"bound": "hbm", "achieved": out_rate / 1e9, "peak": PEAK_HBM / 1e9,
-                          "unit": "GB/s", "frac": out_rate / PEAK_HBM,
-                          "avg_launch_us": ms[pkg.K_OUT] * 1e3 / cnt[pkg.K_OUT]},
-    }
+
+    def hbm(nbytes, k):
+        if cnt[k] == 0:
+            return None
+        rate = nbytes / (ms[k] * 1e-3)
+        return {"bound": "hbm", "achieved": rate / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                "frac": rate / PEAK_HBM, "bytes_per_launch": nbytes / cnt[k],
+                "avg_launch_us": ms[k] * 1e3 / cnt[k], "launches_per_forward": int(cnt[k])}
+
+    transforms = {"out_in_transform": hbm(fused_b, pkg.K_OUTIN),
+                  "in_transform": hbm(in_b, pkg.K_IN),
+                  "out_transform": hbm(out_b, pkg.K_OUT)}
     kernel_ms = {pkg.KERNEL_CLASSES[k]: float(ms[k]) for k in range(pkg.K_COUNT)}
 
     # parity spot check + CPU baseline (oracle as checker / reported baseline only)

@@ -163,7 +163,8 @@ int lzhip_get_act_scales(lzhip_handle* h, float* out, int n);
 #define LZHIP_K_GEMM 2      /* 36-way batched MFMA GEMM                        */
 #define LZHIP_K_OUT 3       /* output transform + BN + residual + ReLU         */
 #define LZHIP_K_HEAD 4      /* 1x1 policy/value convolutions                   */
-#define LZHIP_K_COUNT 5
+#define LZHIP_K_OUTIN 5     /* output transform fused with the next input one  */
+#define LZHIP_K_COUNT 6
 
 /* One forward of n device-resident positions with every kernel launch timed
  * individually by the device's own begin/end timestamps.  ms[LZHIP_K_COUNT]

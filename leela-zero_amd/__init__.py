@@ -28,8 +28,9 @@ MOVES = 362
 VALUE_LAYER = 256
 WINOGRAD_ALPHA = 6
 
-K_PACK, K_IN, K_GEMM, K_OUT, K_HEAD, K_COUNT = 0, 1, 2, 3, 4, 5
-KERNEL_CLASSES = ["pack_input", "in_transform", "gemm", "out_transform", "head_conv"]
+K_PACK, K_IN, K_GEMM, K_OUT, K_HEAD, K_OUTIN, K_COUNT = 0, 1, 2, 3, 4, 5, 6
+KERNEL_CLASSES = ["pack_input", "in_transform", "gemm", "out_transform", "head_conv",
+                  "out_in_transform"]
 
 # Every symbol include/lzhip.h declares.
 EXPORTS = [

@@ -385,19 +385,37 @@ private:
                                 m_stream, timer(timed, LZHIP_K_OUT));
     }
 
+    // Layer loop.  Every layer but the last ends in the fused kernel that turns
+    // M_l straight into V_{l+1}; the spatial activation is written only where a
+    // later layer adds it back as a skip connection (layer 0 and every block
+    // output), and by the last layer for the 1x1 heads.
     void enqueue_forward(int n, const float* d_in, float* d_pol, float* d_val, bool timed) {
+        const int nl = (int)m_layers.size();
+        const int Tu = round_up(n * kTilesPerBoard, kGemmBM);
         launch_pack_input<P>(d_in, m_act0.p, n, kInPlanes, m_C0p, m_stream,
                              timer(timed, LZHIP_K_PACK));
-        int cur = 0, mid = 1, nxt = 2;
-        run_conv(0, n, m_act0.p, nullptr, m_act[cur].p, timed);
-        const int nl = (int)m_layers.size();
-        for (int l = 1; l + 1 < nl; l += 2) {
-            run_conv(l, n, m_act[cur].p, nullptr, m_act[mid].p, timed);
-            run_conv(l + 1, n, m_act[mid].p, m_act[cur].p, m_act[nxt].p, timed);
-            const int o = cur; cur = nxt; nxt = o;
+        launch_in_transform<P>(m_act0.p, m_V.p, n, m_C0p, m_Tp, m_stream,
+                               timer(timed, LZHIP_K_IN));
+        int cur = 0, nxt = 1;  // block input (skip) / block output
+        for (int l = 0; l < nl; l++) {
+            Layer& L = m_layers[l];
+            launch_gemm<P>(m_V.p, L.U.p, m_M.p, Tu, m_Tp, L.Cp, m_Fp, m_stream,
+                           timer(timed, LZHIP_K_GEMM));
+            const bool block_end = (l % 2) == 0;      // layer 0 and second convs
+            const P* res = (block_end && l >= 2) ? m_act[cur].p : nullptr;
+            P* out = l == 0 ? m_act[cur].p : m_act[nxt].p;
+            if (l == nl - 1) {
+                launch_out_transform<P>(m_M.p, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n,
+                                        m_Fp, m_Tp, m_stream, timer(timed, LZHIP_K_OUT));
+                launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, m_stream,
+                                    timer(timed, LZHIP_K_HEAD));
+            } else {
+                launch_out_in_transform<P>(m_M.p, res, block_end ? out : nullptr, m_V.p,
+                                           L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, m_Tp,
+                                           m_stream, timer(timed, LZHIP_K_OUTIN));
+            }
+            if (block_end && l >= 2) { const int o = cur; cur = nxt; nxt = o; }
         }
-        launch_head_conv<P>(m_act[cur].p, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, m_stream,
-                            timer(timed, LZHIP_K_HEAD));
     }
 
     float absmax(const P* x, size_t count) {

@@ -49,6 +49,14 @@ void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scal
                           const float* bn_mean, float rfac, int n, int Kp, int Tp,
                           hipStream_t s, LaunchTimer* t);
 
+// Output transform of one layer fused with the input transform of the next:
+// M [36][Tp][Kp] -> V_next [36][Tp][Kp]; the activation [n][361][Kp] is also
+// written to act_out unless that is null.  Needs Kp to be a multiple of 64.
+template <typename P>
+void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
+                             const float* bn_mean, float rfac, int n, int Kp, int Tp,
+                             hipStream_t s, LaunchTimer* t);
+
 // 1x1 head convolutions: act [n][361][Cp] x w[3][Cp] -> pol [n][2][361], val [n][361],
 // both multiplied by out_scale.
 template <typename P>

@@ -144,13 +144,13 @@ __global__ __launch_bounds__(256) void in_transform_k(const P* __restrict__ act,
 #pragma unroll
         for (int xx = 0; xx < 6; xx++) {
             const int y = y0 + yy, x = x0 + xx;
+            // clamped address + select instead of a branch: all 36 loads stay in flight
+            const bool inb = (unsigned)y < (unsigned)kBoard && (unsigned)x < (unsigned)kBoard;
+            const int pt = inb ? y * kBoard + x : 0;
             float tmp[VN];
+            ChanVec<P>::load(base + (size_t)pt * Cp, tmp);
 #pragma unroll
-            for (int v = 0; v < VN; v++) tmp[v] = 0.0f;
-            if ((unsigned)y < (unsigned)kBoard && (unsigned)x < (unsigned)kBoard)
-                ChanVec<P>::load(base + (size_t)(y * kBoard + x) * Cp, tmp);
-#pragma unroll
-            for (int v = 0; v < VN; v++) d[v][yy * 6 + xx] = tmp[v];
+            for (int v = 0; v < VN; v++) d[v][yy * 6 + xx] = inb ? tmp[v] : 0.0f;
         }
     }
 #pragma unroll
@@ -208,12 +208,12 @@ __global__ __launch_bounds__(256) void out_transform_k(
     const int by = j / 5, bx = j - by * 5;
 
     float m[VN][36];
-    const P* min = M + (size_t)t * Kp + c;
+    const P* msrc = M + (size_t)t * Kp + c;
     const size_t pstride = (size_t)Tp * Kp;
 #pragma unroll
     for (int p = 0; p < 36; p++) {
         float tmp[VN];
-        ChanVec<P>::load(min + p * pstride, tmp);
+        ChanVec<P>::load(msrc + p * pstride, tmp);
 #pragma unroll
         for (int v = 0; v < VN; v++) m[v][p] = tmp[v];
     }
@@ -238,26 +238,36 @@ __global__ __launch_bounds__(256) void out_transform_k(
         mn[v] = bn_mean[c + v];
     }
     const size_t bbase = (size_t)b * kPts * Kp + c;
+    float r[VN][16];
+    if (res != nullptr) {  // uniform; clamped addresses keep the 16 loads free of branches
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                const int y = min(4 * by + i, kBoard - 1), x = min(4 * bx + jj, kBoard - 1);
+                float tmp[VN];
+                ChanVec<P>::load(res + bbase + (size_t)(y * kBoard + x) * Kp, tmp);
+#pragma unroll
+                for (int v = 0; v < VN; v++) r[v][i * 4 + jj] = tmp[v];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < VN; v++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) r[v][q] = 0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
             const int y = 4 * by + i, x = 4 * bx + jj;
-            if (y < kBoard && x < kBoard) {
-                const size_t idx = bbase + (size_t)(y * kBoard + x) * Kp;
-                float val[VN];
+            float val[VN];
 #pragma unroll
-                for (int v = 0; v < VN; v++) val[v] = sc[v] * (o[v][i * 4 + jj] - mn[v]);
-                if (res != nullptr) {
-                    float r[VN];
-                    ChanVec<P>::load(res + idx, r);
-#pragma unroll
-                    for (int v = 0; v < VN; v++) val[v] = val[v] + rfac * r[v];
-                }
-#pragma unroll
-                for (int v = 0; v < VN; v++) val[v] = fmaxf(0.0f, val[v]);
-                ChanVec<P>::store(out + idx, val);
-            }
+            for (int v = 0; v < VN; v++)
+                val[v] = fmaxf(0.0f, sc[v] * (o[v][i * 4 + jj] - mn[v]) + rfac * r[v][i * 4 + jj]);
+            if (y < kBoard && x < kBoard)
+                ChanVec<P>::store(out + bbase + (size_t)(y * kBoard + x) * Kp, val);
         }
     }
 }
@@ -270,6 +280,121 @@ void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scal
     const int lanes = T * (Kp / ChanVec<P>::N);
     launch(out_transform_k<P>, dim3((lanes + 255) / 256), dim3(256), s, t, M, res, out,
            bn_scale, bn_mean, rfac, T, Kp, Tp);
+}
+
+// ---------------------------------------------------------------------------
+// Output transform of layer l fused with the input transform of layer l+1
+// (the reference fuses the same pair for batch 1 only,
+// src/kernels/convolve3.opencl:320-452).  One workgroup owns one board and 64
+// channels: phase 1 turns the 25 M tiles into the 19x19 activation plane
+// (BN, residual, ReLU, rounded to the storage type exactly as the unfused
+// kernel stores it) and keeps it in LDS; phase 2 reads the 6x6 patches back
+// from LDS and writes the next layer's V.  The activation itself goes to
+// memory only when a later layer needs it as a skip connection.
+// Lane = channel, wavefront = tile, so every global access of a wavefront is
+// one contiguous run of 64 channels.
+constexpr int kFuseCG = 64;      // channels per workgroup
+constexpr int kFuseWaves = 12;   // wavefronts per workgroup (3 per SIMD: 168 registers each)
+
+template <typename P>
+__global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
+    const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ act_out,
+    P* __restrict__ Vn, const float* __restrict__ bn_scale, const float* __restrict__ bn_mean,
+    float rfac, int Kp, int Tp) {
+    __shared__ P ybuf[kPts * kFuseCG];
+    const int ncg = Kp / kFuseCG;
+    const int b = blockIdx.x / ncg;
+    const int cg = blockIdx.x - b * ncg;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = cg * kFuseCG + lane;
+    const size_t pstride = (size_t)Tp * Kp;
+    const float sc = bn_scale[c], mn = bn_mean[c];
+
+    // ---- phase 1: A^T m A, BN (+ residual), ReLU -> LDS (+ memory)
+    for (int j = wave; j < kTilesPerBoard; j += kFuseWaves) {
+        const int by = j / 5, bx = j - by * 5;
+        const P* msrc = M + (size_t)(b * kTilesPerBoard + j) * Kp + c;
+        float m[36];
+#pragma unroll
+        for (int p = 0; p < 36; p++) m[p] = (float)msrc[p * pstride];
+        float t1[24], o[16];
+#pragma unroll
+        for (int xx = 0; xx < 6; xx++)
+            at6(m[0 + xx], m[6 + xx], m[12 + xx], m[18 + xx], m[24 + xx], m[30 + xx], t1[0 + xx],
+                t1[6 + xx], t1[12 + xx], t1[18 + xx]);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            at6(t1[i * 6 + 0], t1[i * 6 + 1], t1[i * 6 + 2], t1[i * 6 + 3], t1[i * 6 + 4],
+                t1[i * 6 + 5], o[i * 4 + 0], o[i * 4 + 1], o[i * 4 + 2], o[i * 4 + 3]);
+        const size_t bbase = (size_t)b * kPts * Kp + c;
+        float r[16];
+        if (res != nullptr) {  // uniform; clamped addresses, no branch per load
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int y = min(4 * by + i, kBoard - 1), x = min(4 * bx + jj, kBoard - 1);
+                    r[i * 4 + jj] = (float)res[bbase + (size_t)(y * kBoard + x) * Kp];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 16; q++) r[q] = 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                const int y = 4 * by + i, x = 4 * bx + jj;
+                const P sv = to_storage<P>(
+                    fmaxf(0.0f, sc * (o[i * 4 + jj] - mn) + rfac * r[i * 4 + jj]));
+                if (y < kBoard && x < kBoard) {
+                    const int pt = y * kBoard + x;
+                    ybuf[pt * kFuseCG + lane] = sv;
+                    if (act_out != nullptr) act_out[bbase + (size_t)pt * Kp] = sv;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 2: B^T d B of the next layer from the plane in LDS
+    for (int j = wave; j < kTilesPerBoard; j += kFuseWaves) {
+        const int by = j / 5, bx = j - by * 5;
+        const int y0 = 4 * by - 1, x0 = 4 * bx - 1;
+        float d[36];
+#pragma unroll
+        for (int yy = 0; yy < 6; yy++) {
+#pragma unroll
+            for (int xx = 0; xx < 6; xx++) {
+                const int y = y0 + yy, x = x0 + xx;
+                const bool inb = (unsigned)y < (unsigned)kBoard && (unsigned)x < (unsigned)kBoard;
+                const float v = (float)ybuf[(inb ? y * kBoard + x : 0) * kFuseCG + lane];
+                d[yy * 6 + xx] = inb ? v : 0.0f;
+            }
+        }
+        float t1[36];
+#pragma unroll
+        for (int xx = 0; xx < 6; xx++)
+            bt6(d[0 + xx], d[6 + xx], d[12 + xx], d[18 + xx], d[24 + xx], d[30 + xx], t1[0 + xx],
+                t1[6 + xx], t1[12 + xx], t1[18 + xx], t1[24 + xx], t1[30 + xx]);
+#pragma unroll
+        for (int yy = 0; yy < 6; yy++)
+            bt6(t1[yy * 6 + 0], t1[yy * 6 + 1], t1[yy * 6 + 2], t1[yy * 6 + 3], t1[yy * 6 + 4],
+                t1[yy * 6 + 5], d[yy * 6 + 0], d[yy * 6 + 1], d[yy * 6 + 2], d[yy * 6 + 3],
+                d[yy * 6 + 4], d[yy * 6 + 5]);
+        P* vout = Vn + (size_t)(b * kTilesPerBoard + j) * Kp + c;
+#pragma unroll
+        for (int p = 0; p < 36; p++) vout[p * pstride] = to_storage<P>(d[p]);
+    }
+}
+
+template <typename P>
+void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
+                             const float* bn_mean, float rfac, int n, int Kp, int Tp,
+                             hipStream_t s, LaunchTimer* t) {
+    launch(out_in_transform_k<P>, dim3(n * (Kp / kFuseCG)), dim3(kFuseWaves * 64), s, t, M, res,
+           act_out, Vn, bn_scale, bn_mean, rfac, Kp, Tp);
 }
 
 // ---------------------------------------------------------------------------
@@ -306,27 +431,38 @@ template <> struct Mma<float> {
     }
 };
 
-template <typename P, int BM, int BN>
+// Work items are (position, row tile, column tile) triples, column tile fastest.
+// The device hands workgroup b to accelerator die (XCD) b % 8, each die with its
+// own L2, so the item list is cut into 8 contiguous segments and workgroup b
+// takes item (b / 8) of segment (b % 8): all tiles of one position, and the
+// column tiles that share a V row tile, then run on the same die, U_p and the
+// V tile are fetched from memory once and the repeats hit that die's L2.
+template <typename P, int BM, int BN, int NK>
 __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
                                                    const P* __restrict__ U, P* __restrict__ M,
                                                    int Tp, int Cp, int Kp, int tiles_m,
-                                                   int tiles_n) {
+                                                   int tiles_n, int seg) {
     constexpr int EPC = 16 / sizeof(P);   // elements per 16-byte chunk
     constexpr int BK = 128 / sizeof(P);   // contraction extent of one LDS stage
     constexpr int ROW = BK + EPC;         // padded LDS row, in elements (144 bytes)
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int MB = WM / 32, NB = WN / 32;
     constexpr int A_CH = BM * 8 / 256, B_CH = BN * 8 / 256;  // chunks per thread and stage
+    constexpr int CROW = BN + EPC;        // padded row of the staged output tile
+    constexpr int STAGE = (BM + BN) * ROW;
+    constexpr int SMEM = (2 * STAGE > BM * CROW) ? 2 * STAGE : BM * CROW;
     static_assert(MB >= 1 && NB >= 1, "tile too small for a 2x2 wave grid");
 
-    __shared__ __attribute__((aligned(16))) P As[2][BM * ROW];
-    __shared__ __attribute__((aligned(16))) P Bs[2][BN * ROW];
+    __shared__ __attribute__((aligned(16))) P smem[SMEM];
 
-    int bid = blockIdx.x;
-    const int tn = bid % tiles_n;
-    bid /= tiles_n;
-    const int tm = bid % tiles_m;
-    const int p = bid / tiles_m;
+    const int n_items = kPos * tiles_m * tiles_n;
+    const int xcd = blockIdx.x & 7;
+    const int item = xcd * seg + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= seg || item >= n_items) return;
+    const int tn = item % tiles_n;
+    const int rest = item / tiles_n;
+    const int tm = rest % tiles_m;
+    const int p = rest / tiles_m;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wy = wave >> 1, wx = wave & 1;
@@ -341,60 +477,75 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    int4v ra[A_CH], rb[B_CH];
+    // Two register stages: the slice for step kt+2 is requested while step kt is
+    // being multiplied, so two slices per workgroup are in flight.
+    int4v ra[2][A_CH], rb[2][B_CH];
+    (void)Cp;
     const int lrow = tid >> 3, lch = tid & 7;  // row / chunk of this thread's first chunk
 
-    auto gload = [&](int k0) {
+    auto gload = [&](int st, int k0) {
 #pragma unroll
         for (int i = 0; i < A_CH; i++)
-            ra[i] = *reinterpret_cast<const int4v*>(Ag + (size_t)(lrow + i * 32) * Cp + k0 +
-                                                    lch * EPC);
+            ra[st][i] = *reinterpret_cast<const int4v*>(Ag + (size_t)(lrow + i * 32) * Cp + k0 +
+                                                        lch * EPC);
 #pragma unroll
         for (int i = 0; i < B_CH; i++)
-            rb[i] = *reinterpret_cast<const int4v*>(Bg + (size_t)(lrow + i * 32) * Cp + k0 +
-                                                    lch * EPC);
+            rb[st][i] = *reinterpret_cast<const int4v*>(Bg + (size_t)(lrow + i * 32) * Cp + k0 +
+                                                        lch * EPC);
     };
-    auto lstore = [&](int buf) {
+    auto lstore = [&](int st, int buf) {
+        P* As = smem + buf * STAGE;
+        P* Bs = As + BM * ROW;
 #pragma unroll
         for (int i = 0; i < A_CH; i++)
-            *reinterpret_cast<int4v*>(&As[buf][(lrow + i * 32) * ROW + lch * EPC]) = ra[i];
+            *reinterpret_cast<int4v*>(&As[(lrow + i * 32) * ROW + lch * EPC]) = ra[st][i];
 #pragma unroll
         for (int i = 0; i < B_CH; i++)
-            *reinterpret_cast<int4v*>(&Bs[buf][(lrow + i * 32) * ROW + lch * EPC]) = rb[i];
+            *reinterpret_cast<int4v*>(&Bs[(lrow + i * 32) * ROW + lch * EPC]) = rb[st][i];
     };
 
-    const int nk = Cp / BK;
-    gload(0);
-    lstore(0);
+    // NK = Cp / BK is a template argument: the pipeline below is straight-line
+    // code, so the compiler knows exactly which loads are outstanding at each
+    // wait and the slice for step k+2 really stays in flight across step k.
+    gload(0, 0);
+    if (NK > 1) gload(1, BK);
+    lstore(0, 0);
     __syncthreads();
 
     const int frow = lane & 31, fk = (lane >> 5) * EPC;
-    for (int kt = 0; kt < nk; kt++) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) gload((kt + 1) * BK);
+#pragma unroll
+    for (int k = 0; k < NK; k++) {
+        const int h = k & 1;
+        if (k + 2 < NK) {
+            gload(h, (k + 2) * BK);
+            __builtin_amdgcn_sched_barrier(0);  // request the slice before the math starts
+        }
+        const P* As = smem + h * STAGE;
+        const P* Bs = As + BM * ROW;
 #pragma unroll
         for (int kc = 0; kc < 4; kc++) {
             int4v fa[MB], fb[NB];
 #pragma unroll
             for (int i = 0; i < MB; i++)
                 fa[i] = *reinterpret_cast<const int4v*>(
-                    &As[cur][(wy * WM + i * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+                    &As[(wy * WM + i * 32 + frow) * ROW + kc * 2 * EPC + fk]);
 #pragma unroll
             for (int j = 0; j < NB; j++)
                 fb[j] = *reinterpret_cast<const int4v*>(
-                    &Bs[cur][(wx * WN + j * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+                    &Bs[(wx * WN + j * 32 + frow) * ROW + kc * 2 * EPC + fk]);
 #pragma unroll
             for (int i = 0; i < MB; i++)
 #pragma unroll
                 for (int j = 0; j < NB; j++) acc[i][j] = Mma<P>::run(fa[i], fb[j], acc[i][j]);
         }
-        if (kt + 1 < nk) lstore(cur ^ 1);
+        if (k + 1 < NK) lstore(h ^ 1, h ^ 1);
         __syncthreads();
     }
 
     // Accumulator layout of the 32x32 MFMA: register r of lane l holds
-    // row 8*(r/4) + 4*(l/32) + r%4, column l%32.
-    P* Mg = M + ((size_t)p * Tp + (size_t)tm * BM + wy * WM) * Kp + (size_t)tn * BN + wx * WN;
+    // row 8*(r/4) + 4*(l/32) + r%4, column l%32.  The tile is staged through
+    // LDS (all slices have been consumed) so that it leaves in 16-byte pieces,
+    // whole rows at a time.
     const int crow = 4 * (lane >> 5), ccol = lane & 31;
 #pragma unroll
     for (int i = 0; i < MB; i++)
@@ -402,24 +553,55 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
         for (int j = 0; j < NB; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int row = i * 32 + 8 * (r >> 2) + crow + (r & 3);
-                Mg[(size_t)row * Kp + j * 32 + ccol] = to_storage<P>(acc[i][j][r]);
+                const int row = wy * WM + i * 32 + 8 * (r >> 2) + crow + (r & 3);
+                smem[row * CROW + wx * WN + j * 32 + ccol] = to_storage<P>(acc[i][j][r]);
             }
+    __syncthreads();
+    constexpr int CPR = BN / EPC;  // 16-byte chunks per output row
+    P* Mg = M + ((size_t)p * Tp + (size_t)tm * BM) * Kp + (size_t)tn * BN;
+#pragma unroll 4
+    for (int q = tid; q < BM * CPR; q += 256) {
+        const int row = q / CPR, ch = q - row * CPR;
+        *reinterpret_cast<int4v*>(Mg + (size_t)row * Kp + ch * EPC) =
+            *reinterpret_cast<const int4v*>(&smem[row * CROW + ch * EPC]);
+    }
+}
+
+template <typename P, int BN, int NK>
+static void launch_gemm_nk(const P* V, const P* U, P* M, int tiles_m, int Tp, int Cp, int Kp,
+                           hipStream_t s, LaunchTimer* t) {
+    const int tiles_n = Kp / BN;
+    const int n_items = kPos * tiles_m * tiles_n;
+    int seg = (n_items + 7) / 8;
+    seg = (seg + tiles_n - 1) / tiles_n * tiles_n;  // keep the column tiles of a row tile together
+    launch(wino_gemm_k<P, kGemmBM, BN, NK>, dim3(8 * seg), dim3(256), s, t, V, U, M, Tp, Cp, Kp,
+           tiles_m, tiles_n, seg);
+}
+
+// Channel counts are multiples of 64, so the number of 128-byte k-slices is
+// Cp/64 for fp16 and Cp/32 for fp32; counts up to 512 channels are instantiated.
+template <typename P, int BN>
+static void launch_gemm_bn(const P* V, const P* U, P* M, int tiles_m, int Tp, int Cp, int Kp,
+                           hipStream_t s, LaunchTimer* t) {
+    constexpr int BK = 128 / (int)sizeof(P);
+    switch (Cp / BK) {
+#define LZ_NK(N) case N: launch_gemm_nk<P, BN, N>(V, U, M, tiles_m, Tp, Cp, Kp, s, t); return;
+        LZ_NK(1) LZ_NK(2) LZ_NK(3) LZ_NK(4) LZ_NK(5) LZ_NK(6) LZ_NK(7) LZ_NK(8)
+        LZ_NK(10) LZ_NK(12) LZ_NK(14) LZ_NK(16)
+#undef LZ_NK
+        default: break;
+    }
+    // unreachable for supported widths; the pipe checks the width at creation
 }
 
 template <typename P>
 void launch_gemm(const P* V, const P* U, P* M, int Tp_used, int Tp, int Cp, int Kp,
                  hipStream_t s, LaunchTimer* t) {
     const int tiles_m = Tp_used / kGemmBM;
-    if (Kp % 128 == 0) {
-        const int tiles_n = Kp / 128;
-        launch(wino_gemm_k<P, kGemmBM, 128>, dim3(tiles_m * tiles_n * kPos), dim3(256), s, t, V,
-               U, M, Tp, Cp, Kp, tiles_m, tiles_n);
-    } else {
-        const int tiles_n = Kp / 64;
-        launch(wino_gemm_k<P, kGemmBM, 64>, dim3(tiles_m * tiles_n * kPos), dim3(256), s, t, V,
-               U, M, Tp, Cp, Kp, tiles_m, tiles_n);
-    }
+    if (Kp % 128 == 0)
+        launch_gemm_bn<P, 128>(V, U, M, tiles_m, Tp, Cp, Kp, s, t);
+    else
+        launch_gemm_bn<P, 64>(V, U, M, tiles_m, Tp, Cp, Kp, s, t);
 }
 
 // ---------------------------------------------------------------------------
@@ -590,6 +772,9 @@ void launch_heads(const float* pol, const float* val, HeadParams hp, float tempe
                                  LaunchTimer*);                                                \
     template void launch_out_transform<P>(const P*, const P*, P*, const float*, const float*,  \
                                           float, int, int, int, hipStream_t, LaunchTimer*);    \
+    template void launch_out_in_transform<P>(const P*, const P*, P*, P*, const float*,         \
+                                             const float*, float, int, int, int, hipStream_t,  \
+                                             LaunchTimer*);                                    \
     template void launch_head_conv<P>(const P*, const float*, float, float*, float*, int, int, \
                                       hipStream_t, LaunchTimer*);                              \
     template void launch_absmax<P>(const P*, size_t, float*, hipStream_t);
