@@ -85,7 +85,7 @@ public:
         HIP_CHECK(hipStreamCreate(&m_stream));
         m_Fp = round_up(filters, 64);
         m_C0p = 64;
-        m_Tp = round_up(max_batch * kTilesPerBoard, kGemmBM);
+        m_Tp = round_up(max_batch * kTilesPerBoard, kTileRowPad);
         const size_t B = (size_t)max_batch;
         m_din.alloc(B * kInPlanes * kPts);
         m_dpol.alloc(B * 2 * kPts);
@@ -259,7 +259,7 @@ public:
         HIP_CHECK(hipSetDevice(m_device));
         Layer& L = m_layers[layer];
         const int F = m_filters, C = L.C, Cp = L.Cp;
-        const int Tu = round_up(n * kTilesPerBoard, kGemmBM);
+        const int Tu = n * kTilesPerBoard;
         // stage fp32 NCHW planes through the V buffer's tail?  No: use a scratch buffer.
         DevBuf<float> d_planes, d_res, d_sc, d_mn;
         d_planes.alloc((size_t)n * C * kPts);
@@ -377,7 +377,7 @@ private:
     // Activation buffer roles rotate: cur = block input, mid, nxt = block output.
     void run_conv(int l, int n, const P* in, const P* res, P* out, bool timed) {
         Layer& L = m_layers[l];
-        const int Tu = round_up(n * kTilesPerBoard, kGemmBM);
+        const int Tu = n * kTilesPerBoard;
         launch_in_transform<P>(in, m_V.p, n, L.Cp, m_Tp, m_stream, timer(timed, LZHIP_K_IN));
         launch_gemm<P>(m_V.p, L.U.p, m_M.p, Tu, m_Tp, L.Cp, m_Fp, m_stream,
                        timer(timed, LZHIP_K_GEMM));
@@ -391,7 +391,7 @@ private:
     // output), and by the last layer for the 1x1 heads.
     void enqueue_forward(int n, const float* d_in, float* d_pol, float* d_val, bool timed) {
         const int nl = (int)m_layers.size();
-        const int Tu = round_up(n * kTilesPerBoard, kGemmBM);
+        const int Tu = n * kTilesPerBoard;
         launch_pack_input<P>(d_in, m_act0.p, n, kInPlanes, m_C0p, m_stream,
                              timer(timed, LZHIP_K_PACK));
         launch_in_transform<P>(m_act0.p, m_V.p, n, m_C0p, m_Tp, m_stream,

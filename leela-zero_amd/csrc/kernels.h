@@ -20,7 +20,8 @@ constexpr int kPts = 361;
 constexpr int kTilesPerBoard = 25;
 constexpr int kPos = 36;       // 6x6 Winograd positions
 constexpr int kInPlanes = 18;
-constexpr int kGemmBM = 128;   // GEMM tile extent along T; Tp is a multiple of it
+constexpr int kGemmBM = 128;   // row extent of the standard GEMM tile
+constexpr int kTileRowPad = 256;  // V and M row counts (Tp) are multiples of this
 
 // Timing hook: when non-null every launch is bracketed by this event pair
 // (device begin/end timestamps of that launch alone).
@@ -39,9 +40,10 @@ void launch_in_transform(const P* act, P* V, int n, int Cp, int Tp, hipStream_t 
                          LaunchTimer* t);
 
 // M[p][t][k] = sum_c V[p][t][c] * U[p][k][c]
+// T = real tile rows (25 per board); Tp = allocated rows, a multiple of kTileRowPad.
 template <typename P>
-void launch_gemm(const P* V, const P* U, P* M, int Tp_used, int Tp, int Cp, int Kp,
-                 hipStream_t s, LaunchTimer* t);
+void launch_gemm(const P* V, const P* U, P* M, int T, int Tp, int Cp, int Kp, hipStream_t s,
+                 LaunchTimer* t);
 
 // M [36][Tp][Kp] -> out [n][361][Kp]:  max(0, scale*(A^T m A - mean) + rfac*res)
 template <typename P>

@@ -44,6 +44,11 @@ template <> struct ChanVec<half_t> {
 };
 
 template <typename P> __device__ __forceinline__ P to_storage(float v);
+// Four consecutive storage elements as one LDS/global access.
+template <typename P> struct Quad;
+template <> struct Quad<float> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct Quad<_Float16> { typedef _Float16 type __attribute__((ext_vector_type(4))); };
+
 template <> __device__ __forceinline__ float to_storage<float>(float v) { return v; }
 template <> __device__ __forceinline__ half_t to_storage<half_t>(float v) {
     return (half_t)fminf(fmaxf(v, -65504.0f), 65504.0f);
@@ -408,10 +413,21 @@ void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const 
 // Each lane feeds the matrix cores with 16 contiguous bytes of its row:
 //   fp16: one v_mfma_f32_32x32x16_f16 per fragment pair (8 halves per lane)
 //   fp32: four v_mfma_f32_32x32x2_f32 per fragment pair (one float each)
-// Lane l supplies row (l & 31) of the A block / column (l & 31) of the B
-// block, and the upper half-wave supplies the other half of the k-slice; the
-// assignment of k values to MFMA k-slots is the same for A and B, which is
-// all the contraction needs.  Accumulation is fp32 for both storage types.
+// Lane l supplies row (l & 31) of its 32-row block of either operand, and the
+// upper half-wave supplies the other half of the k-slice; the assignment of k
+// values to MFMA k-slots is the same for both operands, which is all the
+// contraction needs.  Accumulation is fp32 for both storage types.
+// Workgroups of different Winograd positions start their walk over the k-slices at
+// different slices (the sum over k may run in any order): at any moment the
+// 128-byte pieces being fetched then spread over whole 512-byte rows instead of
+// all workgroups hitting the same quarter of every row, which would leave most
+// memory channels idle.  The rotation depends on the position only, so a given
+// board sees the same summation order whatever else is in the batch.
+__device__ __forceinline__ int rotated_slice(int k, int rot, int nk) {
+    const int kk = k + rot;
+    return kk >= nk ? kk - nk : kk;
+}
+
 template <typename P> struct Mma;
 template <> struct Mma<half_t> {
     static __device__ __forceinline__ float16v run(int4v a, int4v b, float16v c) {
@@ -507,8 +523,9 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
     // NK = Cp / BK is a template argument: the pipeline below is straight-line
     // code, so the compiler knows exactly which loads are outstanding at each
     // wait and the slice for step k+2 really stays in flight across step k.
-    gload(0, 0);
-    if (NK > 1) gload(1, BK);
+    const int rot = p % NK;
+    gload(0, rotated_slice(0, rot, NK) * BK);
+    if (NK > 1) gload(1, rotated_slice(1, rot, NK) * BK);
     lstore(0, 0);
     __syncthreads();
 
@@ -517,7 +534,7 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
     for (int k = 0; k < NK; k++) {
         const int h = k & 1;
         if (k + 2 < NK) {
-            gload(h, (k + 2) * BK);
+            gload(h, rotated_slice(k + 2, rot, NK) * BK);
             __builtin_amdgcn_sched_barrier(0);  // request the slice before the math starts
         }
         const P* As = smem + h * STAGE;
@@ -536,25 +553,29 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
 #pragma unroll
             for (int i = 0; i < MB; i++)
 #pragma unroll
-                for (int j = 0; j < NB; j++) acc[i][j] = Mma<P>::run(fa[i], fb[j], acc[i][j]);
+                for (int j = 0; j < NB; j++) acc[i][j] = Mma<P>::run(fb[j], fa[i], acc[i][j]);
         }
         if (k + 1 < NK) lstore(h ^ 1, h ^ 1);
         __syncthreads();
     }
 
-    // Accumulator layout of the 32x32 MFMA: register r of lane l holds
-    // row 8*(r/4) + 4*(l/32) + r%4, column l%32.  The tile is staged through
-    // LDS (all slices have been consumed) so that it leaves in 16-byte pieces,
-    // whole rows at a time.
-    const int crow = 4 * (lane >> 5), ccol = lane & 31;
+    // The U block is the MFMA's row operand and the V block its column operand,
+    // so register r of lane l holds output channel 8*(r/4) + 4*(l/32) + r%4 of
+    // tile row l%32: four consecutive channels per lane, which go to the LDS
+    // staging tile (all slices have been consumed) as one 8- or 16-byte write.
+    // From there whole rows leave in 16-byte pieces.
+    const int ccol = 4 * (lane >> 5), crow = lane & 31;
 #pragma unroll
     for (int i = 0; i < MB; i++)
 #pragma unroll
         for (int j = 0; j < NB; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = wy * WM + i * 32 + 8 * (r >> 2) + crow + (r & 3);
-                smem[row * CROW + wx * WN + j * 32 + ccol] = to_storage<P>(acc[i][j][r]);
+            for (int q = 0; q < 4; q++) {
+                typename Quad<P>::type v;
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = to_storage<P>(acc[i][j][q * 4 + e]);
+                *reinterpret_cast<typename Quad<P>::type*>(
+                    &smem[(wy * WM + i * 32 + crow) * CROW + wx * WN + j * 32 + 8 * q + ccol]) = v;
             }
     __syncthreads();
     constexpr int CPR = BN / EPC;  // 16-byte chunks per output row
@@ -567,6 +588,317 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
     }
 }
 
+// Persistent variant for an even number of k-slices.  A workgroup walks
+// through several work items of its die's segment; the global loads of the
+// next item's first two slices are issued while the current item's last two
+// slices are being multiplied, so every workgroup keeps two slices (64 KB at
+// the 128x128 tile) in flight from its first to its last item instead of
+// starting each tile with an empty pipeline.  The finished tile leaves through
+// the LDS stage that the last slice has just vacated.
+template <typename P, int BM, int BN, int NK>
+__global__ __launch_bounds__(256, 2) void wino_gemm_persistent_k(
+    const P* __restrict__ V, const P* __restrict__ U, P* __restrict__ M, int Tp, int Cp, int Kp,
+    int tiles_m, int tiles_n, int seg, int wg_per_xcd) {
+    static_assert(NK >= 2 && (NK % 2) == 0, "needs an even slice count");
+    constexpr int EPC = 16 / sizeof(P);
+    constexpr int BK = 128 / sizeof(P);
+    constexpr int ROW = BK + EPC;
+    constexpr int WM = BM / 2, WN = BN / 2;
+    constexpr int MB = WM / 32, NB = WN / 32;
+    constexpr int A_CH = BM * 8 / 256, B_CH = BN * 8 / 256;
+    constexpr int CROW = BN + EPC;
+    constexpr int STAGE = (BM + BN) * ROW;
+    // output staging fits one vacated stage either whole or in two row halves
+    constexpr int EP_PARTS = (BM * CROW > STAGE) ? 2 : 1;
+    static_assert((BM / EP_PARTS) * CROW <= STAGE, "output staging does not fit a stage");
+    static_assert(EP_PARTS == 1 || WM * 2 == BM, "row halves must coincide with the wave rows");
+
+    __shared__ __attribute__((aligned(16))) P smem[2 * STAGE];
+
+    const int n_items = kPos * tiles_m * tiles_n;
+    const int xcd = blockIdx.x & 7, w = blockIdx.x >> 3;
+    int item = xcd * seg + w;
+    const int last = min(n_items, (xcd + 1) * seg);
+    if (w >= wg_per_xcd || item >= last) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wy = wave >> 1, wx = wave & 1;
+    const int lrow = tid >> 3, lch = tid & 7;
+    const int frow = lane & 31, fk = (lane >> 5) * EPC;
+    const int ccol = 4 * (lane >> 5), crow = lane & 31;
+    (void)Cp;
+
+    // rs = row stride of the operand loads; the look-ahead past a workgroup's last
+    // item uses rs = 0 and one shared address, so that the loads stay
+    // unconditional (the compiler can then count outstanding loads exactly)
+    // without fetching anything real.
+    struct Ptrs { const P* a; const P* b; P* m; size_t rs; int rot; };
+    auto locate = [&](int it) {
+        const int tn = it % tiles_n;
+        const int rest = it / tiles_n;
+        const int tm = rest % tiles_m;
+        const int p = rest / tiles_m;
+        Ptrs r;
+        r.a = V + ((size_t)p * Tp + (size_t)tm * BM) * Cp + (size_t)lrow * Cp + lch * EPC;
+        r.b = U + ((size_t)p * Kp + (size_t)tn * BN) * Cp + (size_t)lrow * Cp + lch * EPC;
+        r.m = M + ((size_t)p * Tp + (size_t)tm * BM) * Kp + (size_t)tn * BN;
+        r.rs = (size_t)Cp;
+        r.rot = p % NK;
+        return r;
+    };
+
+    int4v ra[2][A_CH], rb[2][B_CH];
+    auto gload = [&](int st, const Ptrs& q, int k0) {
+#pragma unroll
+        for (int i = 0; i < A_CH; i++)
+            ra[st][i] = *reinterpret_cast<const int4v*>(q.a + (size_t)(i * 32) * q.rs + k0);
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+            rb[st][i] = *reinterpret_cast<const int4v*>(q.b + (size_t)(i * 32) * q.rs + k0);
+    };
+    auto lstore = [&](int st, int buf) {
+        P* As = smem + buf * STAGE;
+        P* Bs = As + BM * ROW;
+#pragma unroll
+        for (int i = 0; i < A_CH; i++)
+            *reinterpret_cast<int4v*>(&As[(lrow + i * 32) * ROW + lch * EPC]) = ra[st][i];
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+            *reinterpret_cast<int4v*>(&Bs[(lrow + i * 32) * ROW + lch * EPC]) = rb[st][i];
+    };
+
+    Ptrs cur = locate(item);
+    gload(0, cur, rotated_slice(0, cur.rot, NK) * BK);
+    gload(1, cur, rotated_slice(1, cur.rot, NK) * BK);
+    lstore(0, 0);
+    __syncthreads();
+
+    for (;;) {
+        const int nitem = item + wg_per_xcd;
+        const bool has_next = nitem < last;  // uniform
+        Ptrs nxt = locate(has_next ? nitem : item);
+        if (!has_next) {
+            nxt.a = V;
+            nxt.b = U;
+            nxt.rs = 0;
+        }
+
+        float16v acc[MB][NB];
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+#pragma unroll
+        for (int k = 0; k < NK; k++) {
+            const int h = k & 1;
+            if (k + 2 < NK) {
+                gload(h, cur, rotated_slice(k + 2, cur.rot, NK) * BK);
+            } else {
+                gload(h, nxt, rotated_slice(k + 2 - NK, nxt.rot, NK) * BK);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const P* As = smem + h * STAGE;
+            const P* Bs = As + BM * ROW;
+#pragma unroll
+            for (int kc = 0; kc < 4; kc++) {
+                int4v fa[MB], fb[NB];
+#pragma unroll
+                for (int i = 0; i < MB; i++)
+                    fa[i] = *reinterpret_cast<const int4v*>(
+                        &As[(wy * WM + i * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    fb[j] = *reinterpret_cast<const int4v*>(
+                        &Bs[(wx * WN + j * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+#pragma unroll
+                for (int i = 0; i < MB; i++)
+#pragma unroll
+                    for (int j = 0; j < NB; j++)
+                        acc[i][j] = Mma<P>::run(fb[j], fa[i], acc[i][j]);
+            }
+            lstore(h ^ 1, h ^ 1);
+            __syncthreads();
+        }
+
+        // The last slice sat in stage 1, which is free now (stage 0 already holds
+        // the next item's first slice).
+        P* stage = smem + STAGE;
+        constexpr int CPR = BN / EPC;
+        constexpr int PROWS = BM / EP_PARTS;
+#pragma unroll
+        for (int part = 0; part < EP_PARTS; part++) {
+            if (EP_PARTS == 1 || wy == part) {
+#pragma unroll
+                for (int i = 0; i < MB; i++)
+#pragma unroll
+                    for (int j = 0; j < NB; j++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            typename Quad<P>::type v;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) v[e] = to_storage<P>(acc[i][j][q * 4 + e]);
+                            const int row = (EP_PARTS == 1 ? wy * WM : 0) + i * 32 + crow;
+                            *reinterpret_cast<typename Quad<P>::type*>(
+                                &stage[row * CROW + wx * WN + j * 32 + 8 * q + ccol]) = v;
+                        }
+            }
+            __syncthreads();
+#pragma unroll 4
+            for (int q = tid; q < PROWS * CPR; q += 256) {
+                const int row = q / CPR, ch = q - row * CPR;
+                *reinterpret_cast<int4v*>(cur.m + (size_t)(part * PROWS + row) * Kp + ch * EPC) =
+                    *reinterpret_cast<const int4v*>(&stage[row * CROW + ch * EPC]);
+            }
+            __syncthreads();
+        }
+        if (!has_next) break;
+        item = nitem;
+        cur = nxt;
+    }
+}
+
+// Large-tile variant: one workgroup of 8 wavefronts (2 x 4) owns a 256 x 256
+// tile, i.e. all output channels of 256 tiles when the network has 256
+// filters.  Per multiply-add it moves half as many operand bytes from L2 to
+// the compute unit as the 128 x 128 tile, which is what bounds this GEMM (its
+// contraction is only 256 deep); at 64 boards the 7 x 36 tiles fill the 256
+// compute units in a single round.
+template <typename P, int NK>
+__global__ __launch_bounds__(512) void wino_gemm_big_k(const P* __restrict__ V,
+                                                       const P* __restrict__ U,
+                                                       P* __restrict__ M, int Tp, int Cp, int Kp,
+                                                       int tiles_m, int tiles_n, int seg) {
+    constexpr int BM = 256, BN = 256, NT = 512;
+    constexpr int EPC = 16 / sizeof(P);
+    constexpr int BK = 128 / sizeof(P);
+    constexpr int ROW = BK + EPC;
+    constexpr int WM = 128, WN = 64;       // per-wave tile, waves laid out 2 (rows) x 4 (columns)
+    constexpr int MB = WM / 32, NB = WN / 32;
+    constexpr int A_CH = BM * 8 / NT, B_CH = BN * 8 / NT;
+    constexpr int CROW = BN + EPC;
+    constexpr int STAGE = (BM + BN) * ROW;
+    constexpr int EP_PARTS = sizeof(P) == 2 ? 2 : 4;   // output staged through one vacated stage
+    constexpr int PROWS = BM / EP_PARTS;
+    static_assert(PROWS * CROW <= STAGE, "output staging does not fit a stage");
+
+    __shared__ __attribute__((aligned(16))) P smem[2 * STAGE];
+
+    const int n_items = kPos * tiles_m * tiles_n;
+    const int xcd = blockIdx.x & 7;
+    const int item = xcd * seg + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= seg || item >= n_items) return;
+    const int tn = item % tiles_n;
+    const int rest = item / tiles_n;
+    const int tm = rest % tiles_m;
+    const int p = rest / tiles_m;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wy = wave >> 2, wx = wave & 3;
+    const int lrow = tid >> 3, lch = tid & 7;   // 64 rows per pass of the workgroup
+    const P* Ag = V + ((size_t)p * Tp + (size_t)tm * BM + lrow) * Cp + lch * EPC;
+    const P* Bg = U + ((size_t)p * Kp + (size_t)tn * BN + lrow) * Cp + lch * EPC;
+
+    float16v acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    int4v ra[2][A_CH], rb[2][B_CH];
+    auto gload = [&](int st, int k0) {
+#pragma unroll
+        for (int i = 0; i < A_CH; i++)
+            ra[st][i] = *reinterpret_cast<const int4v*>(Ag + (size_t)(i * 64) * Cp + k0);
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+            rb[st][i] = *reinterpret_cast<const int4v*>(Bg + (size_t)(i * 64) * Cp + k0);
+    };
+    auto lstore = [&](int st, int buf) {
+        P* As = smem + buf * STAGE;
+        P* Bs = As + BM * ROW;
+#pragma unroll
+        for (int i = 0; i < A_CH; i++)
+            *reinterpret_cast<int4v*>(&As[(lrow + i * 64) * ROW + lch * EPC]) = ra[st][i];
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+            *reinterpret_cast<int4v*>(&Bs[(lrow + i * 64) * ROW + lch * EPC]) = rb[st][i];
+    };
+
+    const int rot = p % NK;
+    gload(0, rotated_slice(0, rot, NK) * BK);
+    if (NK > 1) gload(1, rotated_slice(1, rot, NK) * BK);
+    lstore(0, 0);
+    __syncthreads();
+
+    const int frow = lane & 31, fk = (lane >> 5) * EPC;
+#pragma unroll
+    for (int k = 0; k < NK; k++) {
+        const int h = k & 1;
+        if (k + 2 < NK) {
+            gload(h, rotated_slice(k + 2, rot, NK) * BK);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const P* As = smem + h * STAGE;
+        const P* Bs = As + BM * ROW;
+#pragma unroll
+        for (int kc = 0; kc < 4; kc++) {
+            int4v fa[MB], fb[NB];
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+                fa[i] = *reinterpret_cast<const int4v*>(
+                    &As[(wy * WM + i * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                fb[j] = *reinterpret_cast<const int4v*>(
+                    &Bs[(wx * WN + j * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+#pragma unroll
+            for (int i = 0; i < MB; i++)
+#pragma unroll
+                for (int j = 0; j < NB; j++) acc[i][j] = Mma<P>::run(fb[j], fa[i], acc[i][j]);
+        }
+        if (k + 1 < NK) lstore(h ^ 1, h ^ 1);
+        __syncthreads();
+    }
+
+    // Output: PROWS rows at a time through LDS, then out in 16-byte pieces.
+    const int ccol = 4 * (lane >> 5), crow = lane & 31;
+    constexpr int CPR = BN / EPC;
+    P* Mg = M + ((size_t)p * Tp + (size_t)tm * BM) * Kp + (size_t)tn * BN;
+#pragma unroll
+    for (int part = 0; part < EP_PARTS; part++) {
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+            const int row0 = wy * WM + i * 32;      // first tile row of this MFMA block
+            if (row0 / PROWS == part) {             // uniform per wave
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        typename Quad<P>::type v;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] = to_storage<P>(acc[i][j][q * 4 + e]);
+                        *reinterpret_cast<typename Quad<P>::type*>(
+                            &smem[(row0 - part * PROWS + crow) * CROW + wx * WN + j * 32 + 8 * q +
+                                  ccol]) = v;
+                    }
+            }
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int q = tid; q < PROWS * CPR; q += NT) {
+            const int row = q / CPR, ch = q - row * CPR;
+            *reinterpret_cast<int4v*>(Mg + (size_t)(part * PROWS + row) * Kp + ch * EPC) =
+                *reinterpret_cast<const int4v*>(&smem[row * CROW + ch * EPC]);
+        }
+        __syncthreads();
+    }
+}
+
 template <typename P, int BN, int NK>
 static void launch_gemm_nk(const P* V, const P* U, P* M, int tiles_m, int Tp, int Cp, int Kp,
                            hipStream_t s, LaunchTimer* t) {
@@ -574,8 +906,15 @@ static void launch_gemm_nk(const P* V, const P* U, P* M, int tiles_m, int Tp, in
     const int n_items = kPos * tiles_m * tiles_n;
     int seg = (n_items + 7) / 8;
     seg = (seg + tiles_n - 1) / tiles_n * tiles_n;  // keep the column tiles of a row tile together
-    launch(wino_gemm_k<P, kGemmBM, BN, NK>, dim3(8 * seg), dim3(256), s, t, V, U, M, Tp, Cp, Kp,
-           tiles_m, tiles_n, seg);
+    if constexpr (NK >= 2 && (NK % 2) == 0 && BN == 128) {
+        // two resident workgroups on each of a die's 32 compute units
+        const int wg_per_xcd = seg < 64 ? seg : 64;
+        launch(wino_gemm_persistent_k<P, kGemmBM, BN, NK>, dim3(8 * wg_per_xcd), dim3(256), s, t,
+               V, U, M, Tp, Cp, Kp, tiles_m, tiles_n, seg, wg_per_xcd);
+    } else {
+        launch(wino_gemm_k<P, kGemmBM, BN, NK>, dim3(8 * seg), dim3(256), s, t, V, U, M, Tp, Cp,
+               Kp, tiles_m, tiles_n, seg);
+    }
 }
 
 // Channel counts are multiples of 64, so the number of 128-byte k-slices is
@@ -594,10 +933,35 @@ static void launch_gemm_bn(const P* V, const P* U, P* M, int tiles_m, int Tp, in
     // unreachable for supported widths; the pipe checks the width at creation
 }
 
+template <typename P, int NK>
+static void launch_gemm_big(const P* V, const P* U, P* M, int tiles_m, int Tp, int Cp, int Kp,
+                            hipStream_t s, LaunchTimer* t) {
+    const int tiles_n = Kp / 256;
+    const int n_items = kPos * tiles_m * tiles_n;
+    int seg = (n_items + 7) / 8;
+    seg = (seg + tiles_n - 1) / tiles_n * tiles_n;
+    launch(wino_gemm_big_k<P, NK>, dim3(8 * seg), dim3(512), s, t, V, U, M, Tp, Cp, Kp, tiles_m,
+           tiles_n, seg);
+}
+
+// T = number of real tile rows (25 per board); Tp (the row count of V and M)
+// must be a multiple of 256.
 template <typename P>
-void launch_gemm(const P* V, const P* U, P* M, int Tp_used, int Tp, int Cp, int Kp,
-                 hipStream_t s, LaunchTimer* t) {
-    const int tiles_m = Tp_used / kGemmBM;
+void launch_gemm(const P* V, const P* U, P* M, int T, int Tp, int Cp, int Kp, hipStream_t s,
+                 LaunchTimer* t) {
+    constexpr int BK = 128 / (int)sizeof(P);
+    const int nk = Cp / BK;
+    // The 256 x 256 tile pays off once its tiles can occupy most of the 256 compute units.
+    const int big_rows = (T + 255) / 256;
+    if (Kp % 256 == 0 && big_rows * (Kp / 256) * kPos >= 160) {
+        switch (nk) {
+#define LZ_BIG(N) case N: launch_gemm_big<P, N>(V, U, M, big_rows, Tp, Cp, Kp, s, t); return;
+            LZ_BIG(1) LZ_BIG(2) LZ_BIG(4) LZ_BIG(8) LZ_BIG(16)
+#undef LZ_BIG
+            default: break;
+        }
+    }
+    const int tiles_m = (T + kGemmBM - 1) / kGemmBM;
     if (Kp % 128 == 0)
         launch_gemm_bn<P, 128>(V, U, M, tiles_m, Tp, Cp, Kp, s, t);
     else

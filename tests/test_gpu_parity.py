@@ -126,6 +126,19 @@ def test_forward_parity(pkg, netgen, orc, blocks, filters, batch, precision):
     pipe.close()
 
 
+@pytest.mark.parametrize("precision", [0, 1])
+@pytest.mark.parametrize("batch", [64, 41, 24])
+def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
+    """256 filters at batch sizes that select the different GEMM tilings (256x256 tiles
+    from 41 boards up, persistent 128x128 tiles below), in both precisions, including a
+    batch whose tile count is not a multiple of any tile height."""
+    print("case: wide 3x256 b%d precision=%d" % (batch, precision), flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 256, 3000, precision, batch)
+    x = netgen.synthetic_inputs(batch, seed=batch)
+    check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=[0, 1, batch // 2, batch - 1])
+    pipe.close()
+
+
 @pytest.mark.parametrize("blocks,filters,batch", [(20, 256, 32), (40, 256, 64)])
 def test_forward_parity_deep_fp16(pkg, netgen, orc, blocks, filters, batch):
     """Configs 2 and 3 at full size; the oracle checks three positions of the batch."""
