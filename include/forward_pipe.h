@@ -23,7 +23,10 @@
 
 #include "lzhip.h"
 
-#ifndef LZHIP_ENGINE_BUILD
+#ifdef LZHIP_ENGINE_BUILD
+#include "ForwardPipe.h"  // the engine's own declarations
+#include "Network.h"      // NetworkHaltException
+#else
 // Thrown out of forward() when the request was woken by drain()
 // (reference src/Network.h:66-67).
 class NetworkHaltException : public std::exception {};
