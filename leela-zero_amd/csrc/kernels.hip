@@ -300,28 +300,73 @@ void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scal
 // one contiguous run of 64 channels.
 constexpr int kFuseCG = 64;      // channels per workgroup
 constexpr int kFuseWaves = 12;   // wavefronts per workgroup (3 per SIMD: 168 registers each)
+constexpr int kPlane = 22;       // LDS plane: 19 points + 1 zero halo before + 2 after
 
+// Everything that selects a tile is wavefront-uniform and kept in scalar
+// registers (readfirstlane); a lane's pointer is stepped from one Winograd
+// position to the next with a single 64-bit add.  The LDS plane carries a
+// zero halo, so the 6x6 patch reads need no bounds handling.
 template <typename P>
 __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
     const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ act_out,
     P* __restrict__ Vn, const float* __restrict__ bn_scale, const float* __restrict__ bn_mean,
     float rfac, int Kp, int Tp) {
-    __shared__ P ybuf[kPts * kFuseCG];
+    __shared__ P ybuf[kPlane * kPlane * kFuseCG];
     const int ncg = Kp / kFuseCG;
     const int b = blockIdx.x / ncg;
     const int cg = blockIdx.x - b * ncg;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int c = cg * kFuseCG + lane;
+    const unsigned lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const size_t pstride = (size_t)Tp * Kp;
-    const float sc = bn_scale[c], mn = bn_mean[c];
+    const float sc = bn_scale[cg * kFuseCG + lane], mn = bn_mean[cg * kFuseCG + lane];
 
-    // ---- phase 1: A^T m A, BN (+ residual), ReLU -> LDS (+ memory)
+    // zero the halo cells of the plane (rows and columns 0, 20, 21): 3 full rows
+    // and 3 cells in each of the 19 rows between them
+    for (int q = wave; q < 3 * kPlane + 3 * kBoard; q += kFuseWaves) {
+        int cell;
+        if (q < 3 * kPlane) {
+            const int row = q < kPlane ? 0 : (q < 2 * kPlane ? kBoard + 1 : kBoard + 2);
+            cell = row * kPlane + (q % kPlane);
+        } else {
+            const int e = q - 3 * kPlane, y = 1 + e / 3, c3 = e % 3;
+            cell = y * kPlane + (c3 == 0 ? 0 : kBoard + c3);
+        }
+        ybuf[cell * kFuseCG + lane] = (P)0.0f;
+    }
+
+    // ---- phase 1: A^T m A, BN (+ residual), ReLU -> LDS plane (+ memory)
     for (int j = wave; j < kTilesPerBoard; j += kFuseWaves) {
         const int by = j / 5, bx = j - by * 5;
-        const P* msrc = M + (size_t)(b * kTilesPerBoard + j) * Kp + c;
         float m[36];
+        {
+            // per-lane pointer stepped from position to position: one 64-bit add each
+            typedef const __attribute__((address_space(1))) P* gptr_t;  // stays a global pointer
+            gptr_t mp = (gptr_t)(M + ((size_t)(b * kTilesPerBoard + j) * Kp + cg * kFuseCG) + lane);
 #pragma unroll
-        for (int p = 0; p < 36; p++) m[p] = (float)msrc[p * pstride];
+            for (int p = 0; p < 36; p++) {
+                m[p] = (float)*mp;
+                mp += pstride;
+                asm volatile("" : "+v"(mp));  // keep it one add per step (no p * stride)
+            }
+        }
+        // board points of this tile, clamped into the board for the (uniform) addresses
+        // offset of the tile's first board point; rows/columns beyond the board are
+        // clamped for the loads and skipped for the stores (all uniform)
+        const size_t brow = ((size_t)b * kPts + (4 * by) * kBoard + 4 * bx) * Kp + cg * kFuseCG;
+        const int ny = min(4, kBoard - 4 * by), nx = min(4, kBoard - 4 * bx);
+        float r[16];
+        if (res != nullptr) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const P* rp = res + brow + (size_t)(min(i, ny - 1) * kBoard) * Kp + lane;
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++)
+                    r[i * 4 + jj] = (float)rp[(size_t)min(jj, nx - 1) * Kp];
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 16; q++) r[q] = 0.0f;
+        }
         float t1[24], o[16];
 #pragma unroll
         for (int xx = 0; xx < 6; xx++)
@@ -331,21 +376,6 @@ __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
         for (int i = 0; i < 4; i++)
             at6(t1[i * 6 + 0], t1[i * 6 + 1], t1[i * 6 + 2], t1[i * 6 + 3], t1[i * 6 + 4],
                 t1[i * 6 + 5], o[i * 4 + 0], o[i * 4 + 1], o[i * 4 + 2], o[i * 4 + 3]);
-        const size_t bbase = (size_t)b * kPts * Kp + c;
-        float r[16];
-        if (res != nullptr) {  // uniform; clamped addresses, no branch per load
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    const int y = min(4 * by + i, kBoard - 1), x = min(4 * bx + jj, kBoard - 1);
-                    r[i * 4 + jj] = (float)res[bbase + (size_t)(y * kBoard + x) * Kp];
-                }
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < 16; q++) r[q] = 0.0f;
-        }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
 #pragma unroll
@@ -353,10 +383,10 @@ __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
                 const int y = 4 * by + i, x = 4 * bx + jj;
                 const P sv = to_storage<P>(
                     fmaxf(0.0f, sc * (o[i * 4 + jj] - mn) + rfac * r[i * 4 + jj]));
-                if (y < kBoard && x < kBoard) {
-                    const int pt = y * kBoard + x;
-                    ybuf[pt * kFuseCG + lane] = sv;
-                    if (act_out != nullptr) act_out[bbase + (size_t)pt * Kp] = sv;
+                if (i < ny && jj < nx) {  // uniform
+                    ybuf[((y + 1) * kPlane + (x + 1)) * kFuseCG + lane] = sv;
+                    if (act_out != nullptr)
+                        (act_out + brow + (size_t)(i * kBoard + jj) * Kp)[lane] = sv;
                 }
             }
         }
@@ -366,18 +396,14 @@ __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
     // ---- phase 2: B^T d B of the next layer from the plane in LDS
     for (int j = wave; j < kTilesPerBoard; j += kFuseWaves) {
         const int by = j / 5, bx = j - by * 5;
-        const int y0 = 4 * by - 1, x0 = 4 * bx - 1;
+        // patch origin (board row 4by-1, column 4bx-1) = plane cell (4by, 4bx)
+        const P* patch = ybuf + ((4 * by) * kPlane + 4 * bx) * kFuseCG + lane;
         float d[36];
 #pragma unroll
-        for (int yy = 0; yy < 6; yy++) {
+        for (int yy = 0; yy < 6; yy++)
 #pragma unroll
-            for (int xx = 0; xx < 6; xx++) {
-                const int y = y0 + yy, x = x0 + xx;
-                const bool inb = (unsigned)y < (unsigned)kBoard && (unsigned)x < (unsigned)kBoard;
-                const float v = (float)ybuf[(inb ? y * kBoard + x : 0) * kFuseCG + lane];
-                d[yy * 6 + xx] = inb ? v : 0.0f;
-            }
-        }
+            for (int xx = 0; xx < 6; xx++)
+                d[yy * 6 + xx] = (float)patch[(yy * kPlane + xx) * kFuseCG];
         float t1[36];
 #pragma unroll
         for (int xx = 0; xx < 6; xx++)
@@ -388,9 +414,14 @@ __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
             bt6(t1[yy * 6 + 0], t1[yy * 6 + 1], t1[yy * 6 + 2], t1[yy * 6 + 3], t1[yy * 6 + 4],
                 t1[yy * 6 + 5], d[yy * 6 + 0], d[yy * 6 + 1], d[yy * 6 + 2], d[yy * 6 + 3],
                 d[yy * 6 + 4], d[yy * 6 + 5]);
-        P* vout = Vn + (size_t)(b * kTilesPerBoard + j) * Kp + c;
+        typedef __attribute__((address_space(1))) P* gwptr_t;
+        gwptr_t vp = (gwptr_t)(Vn + ((size_t)(b * kTilesPerBoard + j) * Kp + cg * kFuseCG) + lane);
 #pragma unroll
-        for (int p = 0; p < 36; p++) vout[p * pstride] = to_storage<P>(d[p]);
+        for (int p = 0; p < 36; p++) {
+            *vp = to_storage<P>(d[p]);
+            vp += pstride;
+            asm volatile("" : "+v"(vp));
+        }
     }
 }
 
