@@ -6,7 +6,10 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
+#include <map>
+#include <tuple>
 #include <stdexcept>
 
 #include "kernels.h"
@@ -107,6 +110,7 @@ public:
     ~HIPPipeImpl() override {
         (void)hipSetDevice(m_device);
         if (m_stream) (void)hipStreamSynchronize(m_stream);
+        clear_graphs();
         for (int i = 0; i < kTimerPool; i++) {
             if (m_ev_start[i]) (void)hipEventDestroy(m_ev_start[i]);
             if (m_ev_stop[i]) (void)hipEventDestroy(m_ev_stop[i]);
@@ -172,7 +176,7 @@ public:
         std::lock_guard<std::mutex> lk(m_mu);
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
-        enqueue_forward(n, d_in, d_pol, d_val, false);
+        run_forward(n, d_in, d_pol, d_val);
         HIP_CHECK(hipGetLastError());
     }
 
@@ -188,7 +192,7 @@ public:
         std::memcpy(m_hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
         HIP_CHECK(hipMemcpyAsync(m_din.p, m_hin.p, sizeof(float) * (size_t)n * kInPlanes * kPts,
                                  hipMemcpyHostToDevice, m_stream));
-        enqueue_forward(n, m_din.p, m_dpol.p, m_dval.p, false);
+        run_forward(n, m_din.p, m_dpol.p, m_dval.p);
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipMemcpyAsync(m_hpol.p, m_dpol.p, sizeof(float) * (size_t)n * 2 * kPts,
                                  hipMemcpyDeviceToHost, m_stream));
@@ -233,7 +237,7 @@ public:
         HIP_CHECK(hipSetDevice(m_device));
         HIP_CHECK(hipMemcpyAsync(m_din.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts,
                                  hipMemcpyHostToDevice, m_stream));
-        enqueue_forward(n, m_din.p, m_dpol.p, m_dval.p, false);
+        run_forward(n, m_din.p, m_dpol.p, m_dval.p);
         HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
                       m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
         launch_heads(m_dpol.p, m_dval.p, hp, temperature, m_dpolicy.p, m_dlogits.p, m_dvalue.p,
@@ -385,6 +389,39 @@ private:
                                 m_stream, timer(timed, LZHIP_K_OUT));
     }
 
+    // With LZHIP_GRAPH=1 the 165 launches of a forward are captured once per
+    // (batch size, buffers) into a HIP graph and replayed, which takes the launch
+    // work off the host thread.  Only kernel nodes are captured (no memsets or
+    // copies).  On the device the replay measured no faster than stream launches
+    // (the gaps between these kernels are drain and cache write-back, not launch
+    // latency), so plain stream launches are the default.
+    typedef std::tuple<int, const float*, float*, float*> GraphKey;
+    void clear_graphs() {
+        for (auto& kv : m_graphs) (void)hipGraphExecDestroy(kv.second);
+        m_graphs.clear();
+    }
+    void run_forward(int n, const float* d_in, float* d_pol, float* d_val) {
+        if (!m_use_graph) {
+            enqueue_forward(n, d_in, d_pol, d_val, false);
+            return;
+        }
+        const GraphKey key(n, d_in, d_pol, d_val);
+        auto it = m_graphs.find(key);
+        if (it == m_graphs.end()) {
+            if (m_graphs.size() >= 64) clear_graphs();
+            hipGraph_t g = nullptr;
+            hipGraphExec_t ge = nullptr;
+            HIP_CHECK(hipStreamBeginCapture(m_stream, hipStreamCaptureModeThreadLocal));
+            enqueue_forward(n, d_in, d_pol, d_val, false);
+            HIP_CHECK(hipStreamEndCapture(m_stream, &g));
+            const hipError_t e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(g);
+            HIP_CHECK(e);
+            it = m_graphs.emplace(key, ge).first;
+        }
+        HIP_CHECK(hipGraphLaunch(it->second, m_stream));
+    }
+
     // Layer loop.  Every layer but the last ends in the fused kernel that turns
     // M_l straight into V_{l+1}; the spatial activation is written only where a
     // later layer adds it back as a skip connection (layer 0 and every block
@@ -513,6 +550,8 @@ private:
     int m_timer_class[kTimerPool] = {};
     int m_timer_used = 0;
     LaunchTimer m_timer;
+    std::map<GraphKey, hipGraphExec_t> m_graphs;
+    bool m_use_graph = std::getenv("LZHIP_GRAPH") != nullptr;
 };
 
 std::unique_ptr<HIPPipe> create_hip_pipe(int device, int precision, int max_batch, int filters) {

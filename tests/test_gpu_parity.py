@@ -251,3 +251,39 @@ def test_device_resident_forward_and_profile(pkg, netgen, orc):
     assert np.all(ms > 0) and np.all(ms < 50)
     assert np.array_equal(d_pol.cpu().numpy(), pol_h)
     pipe.close()
+
+
+def test_graph_replays_match_stream_launches(pkg, netgen, orc):
+    """The forward is replayed from a captured HIP graph.  Replays of several graphs
+    (different batch sizes and buffers), with other work and synchronisations in between,
+    must reproduce the first results bit for bit, and match a pipe that launches every
+    kernel on the stream (the default; graphs are enabled with LZHIP_GRAPH=1)."""
+    import os
+    import torch
+    _, plain, _, _ = make_pipes(pkg, netgen, orc, 3, 64, 81, pkg.FP16, 8)
+    os.environ["LZHIP_GRAPH"] = "1"
+    try:
+        net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 64, 81, pkg.FP16, 8)
+    finally:
+        del os.environ["LZHIP_GRAPH"]
+    x = netgen.synthetic_inputs(8, seed=9)
+    want8 = plain.forward_batch(x)
+    want3 = plain.forward_batch(x[:3])
+    d_in = torch.from_numpy(x).cuda()
+    d_pol = torch.zeros(8, 722, device="cuda")
+    d_val = torch.zeros(8, 361, device="cuda")
+    for rep in range(4):
+        got8 = pipe.forward_batch(x)                      # graph (8, internal buffers)
+        assert np.array_equal(got8[0], want8[0]) and np.array_equal(got8[1], want8[1]), rep
+        got3 = pipe.forward_batch(x[:3])                  # graph (3, internal buffers)
+        assert np.array_equal(got3[0], want3[0]) and np.array_equal(got3[1], want3[1]), rep
+        d_pol.zero_()
+        torch.cuda.synchronize()
+        pipe.forward_batch_device(8, d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
+        pipe.sync()                                       # graph (8, caller buffers)
+        assert np.array_equal(d_pol.cpu().numpy(), want8[0]), rep
+        assert np.array_equal(d_val.cpu().numpy(), want8[1]), rep
+        policy, value, _ = pipe.evaluate_batch(x[:5])     # eager head kernel after a graph
+        assert policy.shape == (5, 362)
+    pipe.close()
+    plain.close()
