@@ -290,103 +290,224 @@ void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scal
 // ---------------------------------------------------------------------------
 // Output transform of layer l fused with the input transform of layer l+1
 // (the reference fuses the same pair for batch 1 only,
-// src/kernels/convolve3.opencl:320-452).  One workgroup owns one board and 64
-// channels: phase 1 turns the 25 M tiles into the 19x19 activation plane
-// (BN, residual, ReLU, rounded to the storage type exactly as the unfused
-// kernel stores it) and keeps it in LDS; phase 2 reads the 6x6 patches back
-// from LDS and writes the next layer's V.  The activation itself goes to
-// memory only when a later layer needs it as a skip connection.
-// Lane = channel, wavefront = tile, so every global access of a wavefront is
-// one contiguous run of 64 channels.
+// src/kernels/convolve3.opencl:320-452).  Phase 1 turns the 25 M tiles of a
+// board into the 19x19 activation plane (BN, residual, ReLU, rounded to the
+// storage type exactly as the unfused kernel stores it) and keeps it in LDS;
+// phase 2 reads the 6x6 patches back from LDS and writes the next layer's V.
+// The activation itself goes to memory only when a later layer needs it as a
+// skip connection.
+//
+// Raw buffer access: address = buffer base + scalar byte offset + per-lane byte
+// offset.  Everything that selects a board, a tile pair or a Winograd position
+// is wavefront-uniform and lives in the scalar offset, stepped with scalar
+// adds; the per-lane offset never changes, so the global accesses need no
+// vector address arithmetic, and accesses past the end of a buffer are benign.
+template <typename P> struct BufIO;
+template <> struct BufIO<float> {
+    static __device__ __forceinline__ float load(__amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                 unsigned soff) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+    }
+    static __device__ __forceinline__ void store(float v, __amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                 unsigned soff) {
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
+    }
+};
+template <> struct BufIO<half_t> {
+    static __device__ __forceinline__ half_t load(__amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                  unsigned soff) {
+        return __builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0));
+    }
+    static __device__ __forceinline__ void store(half_t v, __amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                 unsigned soff) {
+        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), r, voff, soff,
+                                              0);
+    }
+};
+// Two consecutive channels per access (4 bytes in fp16, 8 in fp32).
+template <typename P> struct BufIO2;
+template <> struct BufIO2<float> {
+    typedef float pair_t __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                unsigned soff, float& a, float& b) {
+        // two 4-byte loads: this compiler lowers the 8-byte raw buffer load builtin
+        // to a single dword load
+        a = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+        b = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff + 4, soff, 0));
+    }
+    static __device__ __forceinline__ void store(pair_t v, __amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                 unsigned soff) {
+        typedef unsigned u2 __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u2, v), r, voff, soff, 0);
+    }
+};
+template <> struct BufIO2<half_t> {
+    typedef half2v pair_t;
+    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                unsigned soff, float& a, float& b) {
+        const half2v h =
+            __builtin_bit_cast(half2v, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+        a = (float)h.x;
+        b = (float)h.y;
+    }
+    static __device__ __forceinline__ void store(pair_t v, __amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                 unsigned soff) {
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
+    }
+};
+
+template <typename P>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const P* base, size_t bytes) {
+    // untyped 32-bit-element descriptor for gfx9-family raw buffer instructions
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<P*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// Stored activations are kept below 65504 / 30.6 (30.6 = largest absolute row
+// sum of B^T (x) B^T), so the input transform of a stored activation cannot
+// leave the half-precision range and V needs no clamp of its own.
+template <typename P> __device__ __forceinline__ P act_to_storage(float v);
+template <> __device__ __forceinline__ float act_to_storage<float>(float v) { return v; }
+template <> __device__ __forceinline__ half_t act_to_storage<half_t>(float v) {
+    return (half_t)fminf(v, 2040.0f);
+}
+
+// One workgroup owns one board and 64 channels.  A lane owns two consecutive
+// channels (one 4- or 8-byte access instead of two), a half-wave owns a tile,
+// so a wavefront handles two neighbouring tiles at once and the 13 wavefronts
+// cover the 25 tiles in a single pass: every wavefront issues its 36 M loads
+// once, up front, instead of walking through several tiles with a full memory
+// latency each, and the number of memory instructions (which bounded the
+// one-channel-per-lane version) is halved.  The two tiles of a wavefront are
+// adjacent rows of M and V, so the half-wave only adds a constant to the lane
+// offset.  The LDS plane carries a zero halo: the 6x6 patch reads need no
+// bounds handling.  Loads that fall outside the board (clipped tiles) read
+// neighbouring memory or, past the end of the buffer, zero (raw buffer
+// semantics); their results are never stored.
 constexpr int kFuseCG = 64;      // channels per workgroup
-constexpr int kFuseWaves = 12;   // wavefronts per workgroup (3 per SIMD: 168 registers each)
+constexpr int kFuseWaves = 13;   // 13 x 2 half-waves >= 25 tiles
 constexpr int kPlane = 22;       // LDS plane: 19 points + 1 zero halo before + 2 after
 
-// Everything that selects a tile is wavefront-uniform and kept in scalar
-// registers (readfirstlane); a lane's pointer is stepped from one Winograd
-// position to the next with a single 64-bit add.  The LDS plane carries a
-// zero halo, so the 6x6 patch reads need no bounds handling.
 template <typename P>
 __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
     const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ act_out,
     P* __restrict__ Vn, const float* __restrict__ bn_scale, const float* __restrict__ bn_mean,
-    float rfac, int Kp, int Tp) {
-    __shared__ P ybuf[kPlane * kPlane * kFuseCG];
+    float rfac, int n, int Kp, int Tp) {
+    typedef typename BufIO2<P>::pair_t pair_t;
+    __shared__ pair_t ybuf[kPlane * kPlane * (kFuseCG / 2)];
+    constexpr int CP = kFuseCG / 2;   // channel pairs per plane cell
     const int ncg = Kp / kFuseCG;
     const int b = blockIdx.x / ncg;
     const int cg = blockIdx.x - b * ncg;
+
     const unsigned lane = threadIdx.x & 63;
+    const unsigned cl = lane & 31, sub = lane >> 5;    // channel pair, tile of the pair
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const size_t pstride = (size_t)Tp * Kp;
-    const float sc = bn_scale[cg * kFuseCG + lane], mn = bn_mean[cg * kFuseCG + lane];
+    const unsigned esz = (unsigned)sizeof(P);
+    const int j = 2 * wave + (int)sub;                 // this lane's tile
+    const bool valid = j < kTilesPerBoard;
+    const int jc = valid ? j : kTilesPerBoard - 1;
+    const int by = jc / 5, bx = jc - by * 5;
+    const int ny = min(4, kBoard - 4 * by), nx = min(4, kBoard - 4 * bx);
+
+    const unsigned pstride = (unsigned)Tp * (unsigned)Kp * esz;   // bytes between positions
+    const size_t tile_bytes = (size_t)kPos * Tp * Kp * esz;
+    const size_t act_bytes = (size_t)n * kPts * Kp * esz;
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(M, tile_bytes);
+    const __amdgpu_buffer_rsrc_t rV = make_rsrc(Vn, tile_bytes);
+    const __amdgpu_buffer_rsrc_t rR = make_rsrc(res != nullptr ? res : M, act_bytes);
+    const __amdgpu_buffer_rsrc_t rA = make_rsrc(act_out != nullptr ? act_out : Vn, act_bytes);
+    // per-lane byte offsets: channel pair (+ one tile row for the upper half-wave) / tile origin
+    const unsigned voff_t = cl * 2 * esz + (valid ? sub : 0u) * (unsigned)Kp * esz;
+    const unsigned voff_a =
+        cl * 2 * esz + (unsigned)((4 * by) * kBoard + 4 * bx) * (unsigned)Kp * esz;
+    // uniform byte offsets of the wavefront's first tile / of the board
+    const unsigned soff_t =
+        ((unsigned)(b * kTilesPerBoard + 2 * wave) * (unsigned)Kp + cg * kFuseCG) * esz;
+    const unsigned soff_a = ((unsigned)(b * kPts) * (unsigned)Kp + cg * kFuseCG) * esz;
+    float sc[2], mn[2];
+#pragma unroll
+    for (int v = 0; v < 2; v++) {
+        sc[v] = bn_scale[cg * kFuseCG + cl * 2 + v];
+        mn[v] = bn_mean[cg * kFuseCG + cl * 2 + v];
+    }
+
+    // all loads of the pass go out first
+    float m[2][36];
+    {
+        unsigned so = soff_t;
+#pragma unroll
+        for (int p = 0; p < 36; p++) {
+            BufIO2<P>::load(rM, voff_t, so, m[0][p], m[1][p]);
+            so += pstride;
+        }
+    }
+    float r[2][16];
+    if (res != nullptr) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+                BufIO2<P>::load(rR, voff_a,
+                                soff_a + (unsigned)(i * kBoard + jj) * (unsigned)Kp * esz,
+                                r[0][i * 4 + jj], r[1][i * 4 + jj]);
+    } else {
+#pragma unroll
+        for (int v = 0; v < 2; v++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) r[v][q] = 0.0f;
+    }
 
     // zero the halo cells of the plane (rows and columns 0, 20, 21): 3 full rows
-    // and 3 cells in each of the 19 rows between them
-    for (int q = wave; q < 3 * kPlane + 3 * kBoard; q += kFuseWaves) {
-        int cell;
-        if (q < 3 * kPlane) {
-            const int row = q < kPlane ? 0 : (q < 2 * kPlane ? kBoard + 1 : kBoard + 2);
-            cell = row * kPlane + (q % kPlane);
-        } else {
-            const int e = q - 3 * kPlane, y = 1 + e / 3, c3 = e % 3;
-            cell = y * kPlane + (c3 == 0 ? 0 : kBoard + c3);
+    // and 3 cells in each of the 19 rows between them; one cell per half-wave
+    {
+        pair_t zero;
+        zero.x = (P)0.0f;
+        zero.y = (P)0.0f;
+        for (int q = 2 * wave + (int)sub; q < 3 * kPlane + 3 * kBoard; q += 2 * kFuseWaves) {
+            int cell;
+            if (q < 3 * kPlane) {
+                const int row = q < kPlane ? 0 : (q < 2 * kPlane ? kBoard + 1 : kBoard + 2);
+                cell = row * kPlane + (q % kPlane);
+            } else {
+                const int e = q - 3 * kPlane, y = 1 + e / 3, c3 = e % 3;
+                cell = y * kPlane + (c3 == 0 ? 0 : kBoard + c3);
+            }
+            ybuf[cell * CP + cl] = zero;
         }
-        ybuf[cell * kFuseCG + lane] = (P)0.0f;
     }
 
     // ---- phase 1: A^T m A, BN (+ residual), ReLU -> LDS plane (+ memory)
-    for (int j = wave; j < kTilesPerBoard; j += kFuseWaves) {
-        const int by = j / 5, bx = j - by * 5;
-        float m[36];
-        {
-            // per-lane pointer stepped from position to position: one 64-bit add each
-            typedef const __attribute__((address_space(1))) P* gptr_t;  // stays a global pointer
-            gptr_t mp = (gptr_t)(M + ((size_t)(b * kTilesPerBoard + j) * Kp + cg * kFuseCG) + lane);
+    // plane cell of the tile's patch origin (board row 4by-1, column 4bx-1)
+    pair_t* const origin = ybuf + ((4 * by) * kPlane + 4 * bx) * CP + cl;
+    {
+        float o[2][16];
 #pragma unroll
-            for (int p = 0; p < 36; p++) {
-                m[p] = (float)*mp;
-                mp += pstride;
-                asm volatile("" : "+v"(mp));  // keep it one add per step (no p * stride)
-            }
+        for (int v = 0; v < 2; v++) {
+            float t1[24];
+#pragma unroll
+            for (int xx = 0; xx < 6; xx++)
+                at6(m[v][0 + xx], m[v][6 + xx], m[v][12 + xx], m[v][18 + xx], m[v][24 + xx],
+                    m[v][30 + xx], t1[0 + xx], t1[6 + xx], t1[12 + xx], t1[18 + xx]);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                at6(t1[i * 6 + 0], t1[i * 6 + 1], t1[i * 6 + 2], t1[i * 6 + 3], t1[i * 6 + 4],
+                    t1[i * 6 + 5], o[v][i * 4 + 0], o[v][i * 4 + 1], o[v][i * 4 + 2],
+                    o[v][i * 4 + 3]);
         }
-        // board points of this tile, clamped into the board for the (uniform) addresses
-        // offset of the tile's first board point; rows/columns beyond the board are
-        // clamped for the loads and skipped for the stores (all uniform)
-        const size_t brow = ((size_t)b * kPts + (4 * by) * kBoard + 4 * bx) * Kp + cg * kFuseCG;
-        const int ny = min(4, kBoard - 4 * by), nx = min(4, kBoard - 4 * bx);
-        float r[16];
-        if (res != nullptr) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const P* rp = res + brow + (size_t)(min(i, ny - 1) * kBoard) * Kp + lane;
-#pragma unroll
-                for (int jj = 0; jj < 4; jj++)
-                    r[i * 4 + jj] = (float)rp[(size_t)min(jj, nx - 1) * Kp];
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < 16; q++) r[q] = 0.0f;
-        }
-        float t1[24], o[16];
-#pragma unroll
-        for (int xx = 0; xx < 6; xx++)
-            at6(m[0 + xx], m[6 + xx], m[12 + xx], m[18 + xx], m[24 + xx], m[30 + xx], t1[0 + xx],
-                t1[6 + xx], t1[12 + xx], t1[18 + xx]);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            at6(t1[i * 6 + 0], t1[i * 6 + 1], t1[i * 6 + 2], t1[i * 6 + 3], t1[i * 6 + 4],
-                t1[i * 6 + 5], o[i * 4 + 0], o[i * 4 + 1], o[i * 4 + 2], o[i * 4 + 3]);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
 #pragma unroll
             for (int jj = 0; jj < 4; jj++) {
-                const int y = 4 * by + i, x = 4 * bx + jj;
-                const P sv = to_storage<P>(
-                    fmaxf(0.0f, sc * (o[i * 4 + jj] - mn) + rfac * r[i * 4 + jj]));
-                if (i < ny && jj < nx) {  // uniform
-                    ybuf[((y + 1) * kPlane + (x + 1)) * kFuseCG + lane] = sv;
+                pair_t sv;
+                sv.x = act_to_storage<P>(
+                    fmaxf(0.0f, sc[0] * (o[0][i * 4 + jj] - mn[0]) + rfac * r[0][i * 4 + jj]));
+                sv.y = act_to_storage<P>(
+                    fmaxf(0.0f, sc[1] * (o[1][i * 4 + jj] - mn[1]) + rfac * r[1][i * 4 + jj]));
+                if (valid && i < ny && jj < nx) {
+                    origin[((i + 1) * kPlane + (jj + 1)) * CP] = sv;
                     if (act_out != nullptr)
-                        (act_out + brow + (size_t)(i * kBoard + jj) * Kp)[lane] = sv;
+                        BufIO2<P>::store(sv, rA, voff_a,
+                                         soff_a + (unsigned)(i * kBoard + jj) * (unsigned)Kp * esz);
                 }
             }
         }
@@ -394,33 +515,40 @@ __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
     __syncthreads();
 
     // ---- phase 2: B^T d B of the next layer from the plane in LDS
-    for (int j = wave; j < kTilesPerBoard; j += kFuseWaves) {
-        const int by = j / 5, bx = j - by * 5;
-        // patch origin (board row 4by-1, column 4bx-1) = plane cell (4by, 4bx)
-        const P* patch = ybuf + ((4 * by) * kPlane + 4 * bx) * kFuseCG + lane;
-        float d[36];
+    {
+        pair_t raw[36];
 #pragma unroll
         for (int yy = 0; yy < 6; yy++)
+#pragma unroll
+            for (int xx = 0; xx < 6; xx++) raw[yy * 6 + xx] = origin[(yy * kPlane + xx) * CP];
+        pair_t outp[36];
+#pragma unroll
+        for (int v = 0; v < 2; v++) {
+            float d[36], t1[36];
+#pragma unroll
+            for (int q = 0; q < 36; q++) d[q] = (float)(v == 0 ? raw[q].x : raw[q].y);
 #pragma unroll
             for (int xx = 0; xx < 6; xx++)
-                d[yy * 6 + xx] = (float)patch[(yy * kPlane + xx) * kFuseCG];
-        float t1[36];
+                bt6(d[0 + xx], d[6 + xx], d[12 + xx], d[18 + xx], d[24 + xx], d[30 + xx],
+                    t1[0 + xx], t1[6 + xx], t1[12 + xx], t1[18 + xx], t1[24 + xx], t1[30 + xx]);
 #pragma unroll
-        for (int xx = 0; xx < 6; xx++)
-            bt6(d[0 + xx], d[6 + xx], d[12 + xx], d[18 + xx], d[24 + xx], d[30 + xx], t1[0 + xx],
-                t1[6 + xx], t1[12 + xx], t1[18 + xx], t1[24 + xx], t1[30 + xx]);
+            for (int yy = 0; yy < 6; yy++)
+                bt6(t1[yy * 6 + 0], t1[yy * 6 + 1], t1[yy * 6 + 2], t1[yy * 6 + 3],
+                    t1[yy * 6 + 4], t1[yy * 6 + 5], d[yy * 6 + 0], d[yy * 6 + 1], d[yy * 6 + 2],
+                    d[yy * 6 + 3], d[yy * 6 + 4], d[yy * 6 + 5]);
 #pragma unroll
-        for (int yy = 0; yy < 6; yy++)
-            bt6(t1[yy * 6 + 0], t1[yy * 6 + 1], t1[yy * 6 + 2], t1[yy * 6 + 3], t1[yy * 6 + 4],
-                t1[yy * 6 + 5], d[yy * 6 + 0], d[yy * 6 + 1], d[yy * 6 + 2], d[yy * 6 + 3],
-                d[yy * 6 + 4], d[yy * 6 + 5]);
-        typedef __attribute__((address_space(1))) P* gwptr_t;
-        gwptr_t vp = (gwptr_t)(Vn + ((size_t)(b * kTilesPerBoard + j) * Kp + cg * kFuseCG) + lane);
+            for (int q = 0; q < 36; q++) {
+                if (v == 0) outp[q].x = (P)d[q];
+                else outp[q].y = (P)d[q];
+            }
+        }
+        if (valid) {
+            unsigned so = soff_t;
 #pragma unroll
-        for (int p = 0; p < 36; p++) {
-            *vp = to_storage<P>(d[p]);
-            vp += pstride;
-            asm volatile("" : "+v"(vp));
+            for (int p = 0; p < 36; p++) {
+                BufIO2<P>::store(outp[p], rV, voff_t, so);
+                so += pstride;
+            }
         }
     }
 }
@@ -430,7 +558,7 @@ void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const 
                              const float* bn_mean, float rfac, int n, int Kp, int Tp,
                              hipStream_t s, LaunchTimer* t) {
     launch(out_in_transform_k<P>, dim3(n * (Kp / kFuseCG)), dim3(kFuseWaves * 64), s, t, M, res,
-           act_out, Vn, bn_scale, bn_mean, rfac, Kp, Tp);
+           act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
 }
 
 // ---------------------------------------------------------------------------
