@@ -73,6 +73,46 @@ def cpu_baseline(orc, netgen, net, x, seconds_budget=20.0):
     }, (pol, val)
 
 
+def search_workload(args, pkg, netgen):
+    """BASELINE configs[4]: tree search with `threads` search threads driving the
+    scheduler at max batch `batch`; every move `visits` root visits, `moves` moves of
+    self-play from the empty board.  Prints one JSON line of its own."""
+    B, F, blocks = args.batch, args.filters, args.blocks
+    prec = pkg.FP16 if args.precision == "fp16" else pkg.FP32
+    net = netgen.make_network(blocks, F, seed=2025)
+    w, h = netgen.prepare(net)
+    pipe = pkg.HIPScheduler(prec, B, device=0)
+    pipe.initialize(F)
+    pipe.push_weights(6, 18, F, w)
+    cfg = pkg.SearchConfig.default(threads=args.threads, visits=args.visits, moves=args.moves,
+                                   seed=2027, reuse_tree=0 if args.no_tree_reuse else 1)
+    warm = pkg.SearchConfig.default(threads=args.threads, visits=min(200, args.visits), moves=1,
+                                    seed=1)
+    pipe.selfplay(h, warm)
+    pipe.reset_stats()
+    res, moves = pipe.selfplay(h, cfg)
+    pipe.close()
+    fill = res.sched.requests / max(1, res.sched.batch_slots)
+    out = {
+        "metric": "search visits/sec and NN batch-fill ratio (BASELINE configs[4])",
+        "value": res.visits_per_s, "unit": "visits/s", "n_gpus": 1, "steps": res.moves_played,
+        "warmup": 1, "ms_per_step": res.seconds / max(1, res.moves_played) * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 storage, f32 accumulate" if prec == pkg.FP16 else "f32",
+        "data": "synthetic (seeded random weights, self-play from the empty board)",
+        "config": {"workload": "%d search threads, max batch %d, %dx%d %s, %d visits/move, "
+                               "%d moves" % (args.threads, B, blocks, F, args.precision,
+                                             args.visits, res.moves_played)},
+        "batch_fill": fill, "mean_batch": res.sched.requests / max(1, res.sched.batches),
+        "max_batch_seen": res.sched.max_batch_seen, "batches": res.sched.batches,
+        "playouts": res.playouts, "nn_evals": res.evals,
+        "nn_evals_per_s": res.sched.requests / res.seconds,
+        "cache_hits": res.cache_hits, "halted": res.halted, "wasted": res.wasted,
+        "seconds": res.seconds, "moves": moves,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -80,10 +120,17 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--blocks", type=int, default=40)
     ap.add_argument("--filters", type=int, default=256)
-    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--batch", type=int, default=None,
+                    help="max batch: default 64 (forward) or 32 (search)")
     ap.add_argument("--precision", choices=["fp16", "fp32"], default="fp16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-reps", type=int, default=5)
+    ap.add_argument("--workload", choices=["forward", "search"], default="forward",
+                    help="forward: the headline metric; search: BASELINE configs[4]")
+    ap.add_argument("--threads", type=int, default=16, help="search threads (search workload)")
+    ap.add_argument("--visits", type=int, default=1600)
+    ap.add_argument("--moves", type=int, default=20)
+    ap.add_argument("--no-tree-reuse", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (one replica per GPU, no "
@@ -96,6 +143,11 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
+    if args.batch is None:
+        args.batch = 64 if args.workload == "forward" else 32
+    if args.workload == "search":
+        search_workload(args, pkg, netgen)
+        return
 
     B, F, blocks = args.batch, args.filters, args.blocks
     prec = pkg.FP16 if args.precision == "fp16" else pkg.FP32

@@ -41,6 +41,13 @@ EXPORTS = [
     "lzhip_debug_layer", "lzhip_get_act_scales", "lzhip_profile_forward", "lzhip_last_error",
     "lzhip_version",
 ]
+# Every symbol include/lzhip_search.h declares.
+SEARCH_EXPORTS = [
+    "lzhip_symmetry_index", "lzhip_gather_features", "lzhip_get_output",
+    "lzhip_search_default_config", "lzhip_selfplay", "lzhip_board_replay",
+]
+
+BLACK, WHITE, EMPTY, PASS = 0, 1, 2, 361
 
 
 class NetworkHaltException(Exception):
@@ -60,6 +67,46 @@ class Stats(ctypes.Structure):
 _lib = None
 _fp = ctypes.POINTER(ctypes.c_float)
 _fpp = ctypes.POINTER(_fp)
+_u8p = ctypes.POINTER(ctypes.c_uint8)
+_ip = ctypes.POINTER(ctypes.c_int)
+
+
+class CHeadWeights(ctypes.Structure):
+    """lzhip_head_weights of include/lzhip_search.h."""
+    _fields_ = [(n, _fp) for n in ["bn_pol_mean", "bn_pol_scale", "ip_pol_w", "ip_pol_b",
+                                   "bn_val_mean", "bn_val_scale", "ip1_val_w", "ip1_val_b",
+                                   "ip2_val_w", "ip2_val_b"]]
+
+
+class SearchConfig(ctypes.Structure):
+    """lzhip_search_config; SearchConfig.default() holds the engine's defaults."""
+    _fields_ = [("threads", ctypes.c_int), ("visits", ctypes.c_int), ("moves", ctypes.c_int),
+                ("cache_size", ctypes.c_int), ("reuse_tree", ctypes.c_int),
+                ("random_moves", ctypes.c_int), ("virtual_loss", ctypes.c_int),
+                ("puct", ctypes.c_float), ("logpuct", ctypes.c_float),
+                ("logconst", ctypes.c_float), ("fpu_reduction", ctypes.c_float),
+                ("softmax_temp", ctypes.c_float), ("komi", ctypes.c_float),
+                ("seed", ctypes.c_uint64)]
+
+    @classmethod
+    def default(cls, **kw):
+        cfg = cls()
+        _check(lib().lzhip_search_default_config(ctypes.byref(cfg)))
+        for k, v in kw.items():
+            if k not in dict(cls._fields_):
+                raise ValueError("unknown search option %r" % k)
+            setattr(cfg, k, v)
+        return cfg
+
+
+class SearchResult(ctypes.Structure):
+    _fields_ = [("playouts", ctypes.c_uint64), ("wasted", ctypes.c_uint64),
+                ("halted", ctypes.c_uint64), ("evals", ctypes.c_uint64),
+                ("cache_lookups", ctypes.c_uint64), ("cache_hits", ctypes.c_uint64),
+                ("nodes", ctypes.c_uint64), ("seconds", ctypes.c_double),
+                ("visits_per_s", ctypes.c_double), ("moves_played", ctypes.c_int),
+                ("passes_at_end", ctypes.c_int), ("final_score", ctypes.c_float),
+                ("sched", Stats)]
 
 
 def lib():
@@ -100,6 +147,17 @@ def lib():
         L.lzhip_get_act_scales.argtypes = [ctypes.c_void_p, _fp, ctypes.c_int]
         L.lzhip_profile_forward.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 3 + \
             [_fp, ctypes.POINTER(ctypes.c_int)]
+        L.lzhip_symmetry_index.argtypes = [ctypes.c_int, ctypes.c_int]
+        L.lzhip_gather_features.argtypes = [_u8p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _fp]
+        L.lzhip_get_output.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights), _u8p,
+                                       ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float,
+                                       _fp, _fp]
+        L.lzhip_search_default_config.argtypes = [ctypes.POINTER(SearchConfig)]
+        L.lzhip_selfplay.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights),
+                                     ctypes.POINTER(SearchConfig), ctypes.POINTER(SearchResult),
+                                     _ip, ctypes.c_int]
+        L.lzhip_board_replay.argtypes = [_ip, ctypes.c_int, ctypes.c_float, _u8p, _u8p, _ip, _ip,
+                                         _fp]
         _lib = L
     return _lib
 
@@ -136,6 +194,55 @@ def process_bn_var(var):
     w = _f32(var).copy()
     _check(lib().lzhip_process_bn_var(_ptr(w), w.size))
     return w
+
+
+def symmetry_index(symmetry, idx):
+    """Board index read by NN index `idx` under `symmetry` (reference
+    src/Network.cpp:518-531, :968-993)."""
+    r = lib().lzhip_symmetry_index(int(symmetry), int(idx))
+    if r < 0:
+        raise ValueError("symmetry in 0..7 and idx in 0..360 expected")
+    return r
+
+
+def _boards(boards):
+    b = np.ascontiguousarray(boards, dtype=np.uint8).reshape(-1, NPTS)
+    return b, b.ctypes.data_as(_u8p)
+
+
+def gather_features(boards, to_move, symmetry=0):
+    """Network::gather_features (reference src/Network.cpp:935-966): boards
+    [n<=8][361] newest first with BLACK/WHITE/EMPTY -> planes [18][361]."""
+    b, bp = _boards(boards)
+    out = np.empty((INPUT_CHANNELS, NPTS), dtype=np.float32)
+    _check(lib().lzhip_gather_features(bp, b.shape[0], int(to_move), int(symmetry), _ptr(out)))
+    return out
+
+
+def board_replay(moves, komi=7.5):
+    """Replays a move list from the empty board with the driver's Go rules and
+    returns dict(stones[361], legal[362], ko_point, superko, score)."""
+    mv = np.ascontiguousarray(moves, dtype=np.int32).reshape(-1)
+    stones = np.empty(NPTS, dtype=np.uint8)
+    legal = np.empty(MOVES, dtype=np.uint8)
+    ko, sk, score = ctypes.c_int(), ctypes.c_int(), ctypes.c_float()
+    _check(lib().lzhip_board_replay(mv.ctypes.data_as(_ip), mv.size, float(komi),
+                                    stones.ctypes.data_as(_u8p), legal.ctypes.data_as(_u8p),
+                                    ctypes.byref(ko), ctypes.byref(sk), ctypes.byref(score)))
+    return {"stones": stones, "legal": legal.astype(bool), "ko_point": ko.value,
+            "superko": bool(sk.value), "score": score.value}
+
+
+def _c_heads(heads):
+    """(struct, keep-alive arrays) for a HeadWeights-like object."""
+    arrs, c = [], CHeadWeights()
+    for name, size in zip(HeadWeights.FIELDS, HeadWeights.SIZES):
+        a = _f32(getattr(heads, name)).reshape(-1)
+        if a.size != size:
+            raise ValueError("%s must have %d values" % (name, size))
+        arrs.append(a)
+        setattr(c, name, _ptr(a))
+    return c, arrs
 
 
 class ForwardPipeWeights:
@@ -303,6 +410,33 @@ class HIPScheduler:
         if want_raw:
             return policy, value, logits, pol, val
         return policy, value, logits
+
+    # -- callers above forward() ------------------------------------------------
+    def get_output(self, heads, boards, to_move, symmetry=0, temperature=1.0):
+        """Network::get_output_internal for one position (reference
+        src/Network.cpp:811-864): returns (policy[362] in board order, winrate)."""
+        self._need()
+        c, keep = _c_heads(heads)
+        b, bp = _boards(boards)
+        policy = np.empty(MOVES, dtype=np.float32)
+        win = ctypes.c_float()
+        _check(lib().lzhip_get_output(self._h, ctypes.byref(c), bp, b.shape[0], int(to_move),
+                                      int(symmetry), float(temperature), _ptr(policy),
+                                      ctypes.byref(win)))
+        del keep
+        return policy, win.value
+
+    def selfplay(self, heads, cfg):
+        """Multi-threaded tree search self-play against this backend; returns
+        (SearchResult, moves)."""
+        self._need()
+        c, keep = _c_heads(heads)
+        res = SearchResult()
+        moves = (ctypes.c_int * max(int(cfg.moves), 1))()
+        _check(lib().lzhip_selfplay(self._h, ctypes.byref(c), ctypes.byref(cfg), ctypes.byref(res),
+                                    moves, len(moves)))
+        del keep
+        return res, list(moves)[:res.moves_played]
 
     # -- introspection ----------------------------------------------------------
     def debug_layer(self, layer, act_in, res=None):

@@ -13,7 +13,8 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "liblzhip.so")
 
-SOURCES = ["kernels.hip", "hip_pipe.hip", "hip_scheduler.cpp", "c_api.cpp"]
+SOURCES = ["kernels.hip", "hip_pipe.hip", "hip_scheduler.cpp", "goboard.cpp", "search.cpp",
+           "c_api.cpp"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are kept out of the generated code.
 HIP_FLAGS = [

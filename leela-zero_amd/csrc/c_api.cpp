@@ -10,6 +10,8 @@
 #include "forward_pipe.h"
 #include "hip_pipe.h"
 #include "lzhip.h"
+#include "lzhip_search.h"
+#include "search.h"
 
 using namespace lzhip;
 
@@ -241,6 +243,107 @@ int lzhip_profile_forward(lzhip_handle* h, int n, const void* d_in, void* d_pol,
     GUARD_BEGIN
     h->pipe->profile_forward(n, static_cast<const float*>(d_in), static_cast<float*>(d_pol),
                              static_cast<float*>(d_val), ms, launches);
+    return LZHIP_OK;
+    GUARD_END
+}
+
+// ---- callers above forward(): planes, one evaluation, search driver ---------
+
+static bool heads_complete(const lzhip_head_weights* w) {
+    return w && w->bn_pol_mean && w->bn_pol_scale && w->ip_pol_w && w->ip_pol_b && w->bn_val_mean &&
+           w->bn_val_scale && w->ip1_val_w && w->ip1_val_b && w->ip2_val_w && w->ip2_val_b;
+}
+
+int lzhip_symmetry_index(int symmetry, int idx) { return symmetry_index(symmetry, idx); }
+
+int lzhip_gather_features(const uint8_t* boards, int n_boards, int to_move, int symmetry,
+                          float* out) {
+    if (!boards || !out) return fail(LZHIP_EINVAL, "null argument");
+    if (n_boards < 1 || n_boards > go::kHistory || (to_move != LZHIP_BLACK && to_move != LZHIP_WHITE) ||
+        symmetry < 0 || symmetry >= 8)
+        return fail(LZHIP_EINVAL, "n_boards in 1..8, to_move 0/1, symmetry 0..7");
+    const uint8_t* ptr[go::kHistory];
+    for (int h = 0; h < n_boards; h++) ptr[h] = boards + (size_t)h * go::kPoints;
+    gather_features(ptr, n_boards, to_move, symmetry, out);
+    return LZHIP_OK;
+}
+
+int lzhip_get_output(lzhip_handle* h, const lzhip_head_weights* heads, const uint8_t* boards,
+                     int n_boards, int to_move, int symmetry, float softmax_temp, float* policy,
+                     float* winrate) {
+    if (!h || !heads_complete(heads) || !boards || !policy || !winrate)
+        return fail(LZHIP_EINVAL, "null argument");
+    if (!(softmax_temp > 0.0f)) return fail(LZHIP_EINVAL, "softmax_temp must be positive");
+    GUARD_BEGIN
+    std::vector<float> in(LZHIP_INPUT_SIZE), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
+    const int rc = lzhip_gather_features(boards, n_boards, to_move, symmetry, in.data());
+    if (rc != LZHIP_OK) return rc;
+    const int frc = h->sched->forward_raw(in.data(), pol.data(), val.data());
+    if (frc == LZHIP_EHALT) return fail(LZHIP_EHALT, "halted by drain");
+    const HeadWeights hw(*heads);
+    float p[go::kPoints + 1];
+    heads_on_host(hw, pol.data(), val.data(), softmax_temp, p, winrate);
+    for (int i = 0; i < go::kPoints; i++) policy[symmetry_index(symmetry, i)] = p[i];
+    policy[go::kPoints] = p[go::kPoints];
+    return LZHIP_OK;
+    GUARD_END
+}
+
+int lzhip_search_default_config(lzhip_search_config* cfg) {
+    if (!cfg) return fail(LZHIP_EINVAL, "null argument");
+    std::memset(cfg, 0, sizeof(*cfg));
+    cfg->threads = 16;
+    cfg->visits = 1600;
+    cfg->moves = 20;
+    cfg->cache_size = 150000;
+    cfg->reuse_tree = 1;
+    cfg->random_moves = 0;
+    cfg->virtual_loss = 3;
+    cfg->puct = 0.5f;
+    cfg->logpuct = 0.015f;
+    cfg->logconst = 1.7f;
+    cfg->fpu_reduction = 0.25f;
+    cfg->softmax_temp = 1.0f;
+    cfg->komi = 7.5f;
+    cfg->seed = 1;
+    return LZHIP_OK;
+}
+
+int lzhip_selfplay(lzhip_handle* h, const lzhip_head_weights* heads,
+                   const lzhip_search_config* cfg, lzhip_search_result* result, int* moves_out,
+                   int moves_cap) {
+    if (!h || !heads_complete(heads) || !cfg || !result) return fail(LZHIP_EINVAL, "null argument");
+    if (cfg->threads < 1 || cfg->threads > 4096 || cfg->visits < 1 || cfg->moves < 0 ||
+        !(cfg->softmax_temp > 0.0f))
+        return fail(LZHIP_EINVAL, "threads in 1..4096, visits >= 1, moves >= 0, softmax_temp > 0");
+    GUARD_BEGIN
+    selfplay(*h->sched, *heads, *cfg, *result, moves_out, moves_out ? moves_cap : 0);
+    return LZHIP_OK;
+    GUARD_END
+}
+
+int lzhip_board_replay(const int* moves, int n_moves, float komi, uint8_t* stones, uint8_t* legal,
+                       int* ko_point, int* superko, float* score) {
+    if (n_moves < 0 || (n_moves > 0 && !moves)) return fail(LZHIP_EINVAL, "bad move list");
+    GUARD_BEGIN
+    go::Position pos;
+    bool repeated = false;
+    for (int i = 0; i < n_moves; i++) {
+        const int mv = moves[i];
+        if (mv < 0 || mv > go::kPass || !pos.legal_slow(pos.to_move(), mv))
+            return fail(LZHIP_EINVAL, "illegal move in the list");
+        pos.play(mv);
+        repeated = (mv != go::kPass) && pos.superko();
+    }
+    if (stones) std::memcpy(stones, pos.stones().data(), go::kPoints);
+    if (legal) {
+        go::GroupInfo g;
+        pos.analyze(g);
+        for (int v = 0; v <= go::kPass; v++) legal[v] = pos.legal(g, pos.to_move(), v) ? 1 : 0;
+    }
+    if (ko_point) *ko_point = pos.ko_point();
+    if (superko) *superko = repeated ? 1 : 0;
+    if (score) *score = pos.area_score(komi);
     return LZHIP_OK;
     GUARD_END
 }

@@ -1,0 +1,310 @@
+// Host-only test of the search driver against a stand-in executor behind the
+// real batching scheduler; meant to be built plainly and with -fsanitize=thread.
+// The stand-in "network" is equivariant under the eight board symmetries, so a
+// wrong rotation or un-rotation of planes or policy shows up as a wrong prior.
+//
+// Checked, after the call pattern of the reference's search
+// (src/UCTSearch.cpp:237-286, :757-850; src/UCTNode.cpp:62-155, :306-362):
+//   * priors come back in board order for every symmetry;
+//   * every move played is legal, visit budgets are met, and when the threads
+//     have left no virtual loss or half-expanded node remains and every
+//     expanded node holds 1 + the visits of its children;
+//   * requests still queued at the end of a move are released by the halt and
+//     the scheduler answers again afterwards;
+//   * one thread with one seed plays the same game twice;
+//   * the evaluation cache answers repeated positions;
+//   * a finished game (two passes) is not searched;
+//   * an executor failure reaches the caller as an exception.
+#include <atomic>
+#include <chrono>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <stdexcept>
+#include <thread>
+#include <vector>
+
+#include "forward_pipe.h"
+#include "search.h"
+
+using namespace lzhip;
+using go::kPass;
+using go::kPoints;
+
+namespace lzhip {
+std::unique_ptr<BatchExecutor> make_hip_pipe(int, int, int, int) {
+    throw std::runtime_error("no device in the search test");
+}
+}  // namespace lzhip
+
+#define CHECK(cond)                                                                 \
+    do {                                                                            \
+        if (!(cond)) {                                                              \
+            std::fprintf(stderr, "FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            std::exit(1);                                                           \
+        }                                                                           \
+    } while (0)
+
+// pol plane 0 at i = 3 * (opponent stones of the newest board next to i);
+// val plane at i = 1 + own stone - opponent stone at i (newest board).
+class NeighbourNet : public BatchExecutor {
+public:
+    NeighbourNet(int mb, int delay_us) : m_mb(mb), m_delay(delay_us) {}
+    int max_batch() const override { return m_mb; }
+    void forward_batch(int n, const float* in, float* pol, float* val) override {
+        if (fail.load()) throw std::runtime_error("injected failure");
+        if (m_delay) std::this_thread::sleep_for(std::chrono::microseconds(m_delay));
+        for (int b = 0; b < n; b++) {
+            const float* x = in + (size_t)b * LZHIP_INPUT_SIZE;
+            const float* own = x;
+            const float* opp = x + 8 * kPoints;
+            float* p = pol + (size_t)b * LZHIP_POL_SIZE;
+            float* v = val + (size_t)b * LZHIP_VAL_SIZE;
+            for (int i = 0; i < kPoints; i++) {
+                const int xx = i % 19, yy = i / 19;
+                float s = 0.0f;
+                if (xx > 0) s += opp[i - 1];
+                if (xx < 18) s += opp[i + 1];
+                if (yy > 0) s += opp[i - 19];
+                if (yy < 18) s += opp[i + 19];
+                p[i] = 3.0f * s;
+                p[kPoints + i] = 0.0f;
+                v[i] = own[i] - opp[i] + 1.0f;
+            }
+        }
+        batches++;
+        positions += n;
+    }
+    std::atomic<bool> fail{false};
+    std::atomic<long> batches{0}, positions{0};
+
+private:
+    int m_mb, m_delay;
+};
+
+// Heads: logit[o] = pol plane 0 at o (pass logit 0); value = tanh(0.05 * stone
+// difference) for differences above -10 -> the side with more stones is ahead.
+struct Heads {
+    std::vector<float> bn_pol_mean{0, 0}, bn_pol_scale{1, 1}, ip_pol_w, ip_pol_b, bn_val_mean{0},
+        bn_val_scale{1}, ip1_val_w, ip1_val_b, ip2_val_w, ip2_val_b{0};
+    lzhip_head_weights c{};
+    Heads() {
+        ip_pol_w.assign((size_t)362 * 722, 0.0f);
+        for (int o = 0; o < kPoints; o++) ip_pol_w[(size_t)o * 722 + o] = 1.0f;
+        ip_pol_b.assign(362, 0.0f);
+        ip1_val_w.assign((size_t)256 * kPoints, 0.0f);
+        for (int i = 0; i < kPoints; i++) ip1_val_w[i] = 1.0f;
+        ip1_val_b.assign(256, 0.0f);
+        ip1_val_b[0] = -351.0f;  // hidden unit 0 = relu(10 + own - opp)
+        ip2_val_w.assign(256, 0.0f);
+        ip2_val_w[0] = 0.05f;
+        ip2_val_b[0] = -0.5f;
+        c.bn_pol_mean = bn_pol_mean.data();
+        c.bn_pol_scale = bn_pol_scale.data();
+        c.ip_pol_w = ip_pol_w.data();
+        c.ip_pol_b = ip_pol_b.data();
+        c.bn_val_mean = bn_val_mean.data();
+        c.bn_val_scale = bn_val_scale.data();
+        c.ip1_val_w = ip1_val_w.data();
+        c.ip1_val_b = ip1_val_b.data();
+        c.ip2_val_w = ip2_val_w.data();
+        c.ip2_val_b = ip2_val_b.data();
+    }
+};
+
+static lzhip_search_config config(int threads, int visits, int moves) {
+    lzhip_search_config c{};
+    c.threads = threads;
+    c.visits = visits;
+    c.moves = moves;
+    c.cache_size = 20000;
+    c.reuse_tree = 1;
+    c.random_moves = 0;
+    c.virtual_loss = 3;
+    c.puct = 0.5f;
+    c.logpuct = 0.015f;
+    c.logconst = 1.7f;
+    c.fpu_reduction = 0.25f;
+    c.softmax_temp = 1.0f;
+    c.komi = 7.5f;
+    c.seed = 7;
+    return c;
+}
+
+static void test_unrotation() {
+    HIPScheduler sched(std::make_unique<NeighbourNet>(4, 0));
+    Heads heads;
+    NetworkFacade net(sched, heads.c, 0, 1.0f);
+    go::Position pos;
+    const int stone = 5 * 19 + 2;  // (2,5): off every symmetry axis
+    pos.play(stone);               // black; white to move sees one opponent stone
+    uint64_t rng = 99;
+    for (int sym = 0; sym < 8; sym++) {
+        const Netresult r = net.get_output(pos, sym, rng, false);
+        // the four neighbours of the stone share the top prior, in board order
+        const float top = r.policy[stone - 1];
+        CHECK(top > 0.04f);
+        CHECK(std::fabs(r.policy[stone + 1] - top) < 1e-6f);
+        CHECK(std::fabs(r.policy[stone - 19] - top) < 1e-6f);
+        CHECK(std::fabs(r.policy[stone + 19] - top) < 1e-6f);
+        int above = 0;
+        for (int i = 0; i < kPoints; i++)
+            if (r.policy[i] > top * 0.5f) above++;
+        CHECK(above == 4);
+        CHECK(r.winrate < 0.5f);  // the side to move is a stone behind
+        float sum = r.policy_pass;
+        for (int i = 0; i < kPoints; i++) sum += r.policy[i];
+        CHECK(std::fabs(sum - 1.0f) < 1e-4f);
+    }
+}
+
+static std::vector<int> play_game(int threads, int visits, int moves, int delay_us, int max_batch,
+                                  lzhip_search_result* res_out, int reuse = 1) {
+    HIPScheduler sched(std::make_unique<NeighbourNet>(max_batch, delay_us));
+    Heads heads;
+    lzhip_search_config cfg = config(threads, visits, moves);
+    cfg.reuse_tree = reuse;
+    NetworkFacade net(sched, heads.c, (size_t)cfg.cache_size, 1.0f);
+    UCTSearch search(net, cfg);
+    go::Position pos;
+    std::vector<int> game;
+    for (int m = 0; m < moves && pos.passes() < 2; m++) {
+        const int before = search.root_visits();
+        const int mv = search.think(pos);
+        CHECK(search.root_visits() >= visits);
+        CHECK(search.root_visits() >= before);
+        const auto tc = search.check_tree();
+        CHECK(tc.virtual_loss == 0);
+        CHECK(tc.expanding == 0);
+        CHECK(tc.visit_mismatch == 0);
+        CHECK(mv == kPass || pos.legal_slow(pos.to_move(), mv));
+        // the chosen move is the most visited child
+        int best = -1;
+        for (auto& cv : search.root_children()) best = std::max(best, cv.second);
+        for (auto& cv : search.root_children())
+            if (cv.first == mv) CHECK(cv.second == best);
+        pos.play(mv);
+        CHECK(!(mv != kPass && pos.superko()));
+        search.advance(mv);
+        game.push_back(mv);
+    }
+    // the backend answers again after the halts
+    std::vector<float> in(LZHIP_INPUT_SIZE, 0.0f), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
+    sched.forward(in, pol, val);
+    if (res_out) {
+        res_out->playouts = search.stats().playouts;
+        res_out->halted = search.stats().halted;
+        res_out->wasted = search.stats().wasted;
+        res_out->evals = net.evals();
+        res_out->cache_hits = net.cache().hits();
+        res_out->cache_lookups = net.cache().lookups();
+        res_out->sched = sched.stats();
+    }
+    return game;
+}
+
+static void test_single_thread_deterministic() {
+    lzhip_search_result a{}, b{};
+    const auto g1 = play_game(1, 120, 6, 0, 4, &a);
+    const auto g2 = play_game(1, 120, 6, 0, 4, &b);
+    CHECK(g1 == g2);
+    CHECK(g1.size() == 6);
+    CHECK(a.playouts == b.playouts);
+    CHECK(a.halted <= 6);  // one thread: at most the request in flight at each stop
+    // with the neighbour prior white's first reply touches black's first stone
+    const int d = std::abs(g1[1] - g1[0]);
+    CHECK(d == 1 || d == 19);
+}
+
+static void test_many_threads() {
+    lzhip_search_result r{};
+    const auto g = play_game(12, 300, 5, 150, 8, &r);
+    CHECK(g.size() == 5);
+    CHECK(r.playouts >= 5 * 200);
+    CHECK(r.sched.max_batch_seen <= 8);
+    CHECK(r.sched.max_batch_seen >= 2);  // concurrent requests were batched
+    CHECK(r.sched.requests + r.sched.halted >= r.evals);
+    std::printf("  12 threads: playouts %llu evals %llu halted %llu wasted %llu batches %llu max %u\n",
+                (unsigned long long)r.playouts, (unsigned long long)r.evals,
+                (unsigned long long)r.halted, (unsigned long long)r.wasted,
+                (unsigned long long)r.sched.batches, r.sched.max_batch_seen);
+}
+
+static void test_cache_hits_without_tree_reuse() {
+    lzhip_search_result r{};
+    play_game(2, 150, 3, 0, 4, &r, /*reuse=*/0);
+    CHECK(r.cache_hits > 50);  // the second and third searches revisit known positions
+    CHECK(r.evals + r.cache_hits == r.cache_lookups);
+}
+
+static void test_finished_game_is_not_searched() {
+    HIPScheduler sched(std::make_unique<NeighbourNet>(4, 0));
+    Heads heads;
+    lzhip_search_config cfg = config(2, 50, 1);
+    NetworkFacade net(sched, heads.c, 100, 1.0f);
+    UCTSearch search(net, cfg);
+    go::Position pos;
+    pos.play(kPass);
+    pos.play(kPass);
+    CHECK(search.think(pos) == kPass);
+    CHECK(net.evals() == 0);
+}
+
+static void test_selfplay_entry_and_failure() {
+    Heads heads;
+    {
+        HIPScheduler sched(std::make_unique<NeighbourNet>(8, 50));
+        lzhip_search_config cfg = config(6, 100, 4);
+        lzhip_search_result res;
+        int moves[4] = {-1, -1, -1, -1};
+        selfplay(sched, heads.c, cfg, res, moves, 4);
+        CHECK(res.moves_played == 4);
+        CHECK(res.playouts > 0 && res.seconds > 0 && res.visits_per_s > 0);
+        CHECK(res.sched.batches > 0 && res.sched.batch_slots == res.sched.batches * 8);
+        CHECK(res.sched.requests <= res.evals);
+        for (int m : moves) CHECK(m >= 0 && m <= kPass);
+    }
+    {
+        auto exec = std::make_unique<NeighbourNet>(4, 0);
+        exec->fail = true;
+        HIPScheduler sched(std::move(exec));
+        lzhip_search_config cfg = config(3, 50, 2);
+        lzhip_search_result res;
+        bool threw = false;
+        try {
+            selfplay(sched, heads.c, cfg, res, nullptr, 0);
+        } catch (const std::runtime_error&) {
+            threw = true;
+        }
+        CHECK(threw);
+    }
+    {
+        HIPScheduler sched(std::make_unique<NeighbourNet>(4, 0));
+        lzhip_search_config cfg = config(0, 50, 2);
+        lzhip_search_result res;
+        bool threw = false;
+        try {
+            selfplay(sched, heads.c, cfg, res, nullptr, 0);
+        } catch (const std::invalid_argument&) {
+            threw = true;
+        }
+        CHECK(threw);
+    }
+}
+
+int main() {
+    std::printf("unrotation\n");
+    test_unrotation();
+    std::printf("single thread\n");
+    test_single_thread_deterministic();
+    std::printf("many threads\n");
+    test_many_threads();
+    std::printf("cache\n");
+    test_cache_hits_without_tree_reuse();
+    std::printf("finished game\n");
+    test_finished_game_is_not_searched();
+    std::printf("selfplay entry\n");
+    test_selfplay_entry_and_failure();
+    std::printf("search tests passed\n");
+    return 0;
+}

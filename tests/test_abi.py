@@ -21,6 +21,25 @@ def test_library_exports_every_declared_symbol(pkg):
     assert sorted(pkg.EXPORTS) == declared
 
 
+def test_library_exports_every_search_symbol(pkg):
+    header = open(os.path.join(ROOT, "include", "lzhip_search.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(lzhip_[a-z0-9_]+)\s*\(", header)))
+    assert len(declared) == 6
+    L = ctypes.CDLL(pkg.LIB_PATH)
+    for name in declared:
+        assert hasattr(L, name), name
+    assert sorted(pkg.SEARCH_EXPORTS) == declared
+    # struct sizes the ctypes mirror assumes
+    assert ctypes.sizeof(pkg.SearchConfig) == 64
+    assert ctypes.sizeof(pkg.CHeadWeights) == 80
+    cfg = pkg.SearchConfig.default()
+    assert (cfg.threads, cfg.visits, cfg.moves, cfg.virtual_loss) == (16, 1600, 20, 3)
+    assert abs(cfg.puct - 0.5) < 1e-7 and abs(cfg.komi - 7.5) < 1e-7
+    assert L.lzhip_selfplay(None, None, None, None, None, 0) == pkg.EINVAL
+    assert L.lzhip_get_output(None, None, None, 1, 0, 0, ctypes.c_float(1.0), None, None) == pkg.EINVAL
+
+
 def test_version_and_error_string(pkg):
     assert "gfx950" in pkg.version()
     assert isinstance(pkg.lib().lzhip_last_error(), bytes)

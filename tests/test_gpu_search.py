@@ -1,0 +1,107 @@
+"""The callers above forward() on the GPU: one full evaluation (planes -> device ->
+heads -> policy in board order) against the oracle chain for every symmetry, and the
+multi-threaded search driver against the real backend (legal games, consistent counters,
+batches formed from concurrent single-position requests)."""
+import numpy as np
+import pytest
+
+import oracle.go_oracle as G
+
+pytestmark = pytest.mark.gpu
+
+
+def make(pkg, netgen, orc, blocks, filters, seed, precision, max_batch):
+    net = netgen.make_network(blocks, filters, seed)
+    w, h = netgen.prepare(net)
+    w_ref, h_ref = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    ref = orc.OraclePipe()
+    ref.initialize(filters)
+    ref.push_weights(6, 18, filters, w_ref)
+    pipe = pkg.HIPScheduler(precision, max_batch)
+    pipe.initialize(filters)
+    pipe.push_weights(6, 18, filters, w)
+    return pipe, h, ref, h_ref
+
+
+def random_position(seed, plies):
+    """A position with captures and a full 8-board history, from the plain-Python rules."""
+    rng = np.random.default_rng(seed)
+    b = G.Board()
+    for _ in range(plies):
+        mask = b.legal_mask()
+        cand = [v for v in range(361) if mask[v]]
+        b.play(int(rng.choice(cand)))
+    boards = [list(p) for p in reversed(b.history[-8:])]   # newest first
+    return b, boards
+
+
+@pytest.mark.parametrize("precision", [0, 1])
+def test_get_output_matches_oracle_chain(pkg, netgen, orc, precision):
+    print("case: get_output precision=%d" % precision, flush=True)
+    pipe, h, ref, h_ref = make(pkg, netgen, orc, 3, 64, 11, precision, 4)
+    tol = 1e-4 if precision == 0 else 2e-2
+    orc.use_builtin()
+    worst = 0.0
+    for seed, plies in ((5, 40), (6, 181)):
+        b, boards = random_position(seed, plies)
+        for sym in range(8):
+            policy, winrate = pipe.get_output(h, np.array(boards, np.uint8), b.to_move, sym)
+            planes = np.array(G.gather_features(boards, b.to_move, sym), np.float32)
+            rp, rv = ref.forward(planes)
+            hd = orc.heads(h_ref, rp, rv)
+            want = np.empty(362, np.float32)
+            for idx in range(361):
+                want[G.symmetry_index(sym, idx)] = hd["policy"][idx]
+            want[361] = hd["policy"][361]
+            err = max(float(np.abs(policy - want).max()), abs(winrate - hd["winrate"]))
+            worst = max(worst, err)
+            assert err <= tol, (seed, sym, err)
+            assert abs(float(policy.sum()) - 1.0) < 1e-4
+    print("get_output worst", worst, flush=True)
+    pipe.close()
+
+
+def test_selfplay_on_device(pkg, netgen, orc):
+    print("case: selfplay 2x64 fp16, 12 threads, batch 8", flush=True)
+    pipe, h, ref, h_ref = make(pkg, netgen, orc, 2, 64, 21, 1, 8)
+    cfg = pkg.SearchConfig.default(threads=12, visits=200, moves=8, seed=3)
+    res, moves = pipe.selfplay(h, cfg)
+    assert res.moves_played == len(moves) == 8
+    # every move is legal under the independent rules and none repeats a position
+    b = G.Board()
+    for mv in moves:
+        assert b.is_legal(b.to_move, mv), mv
+        b.play(mv)
+        assert not (mv != G.PASS and b.superko())
+    assert res.final_score == b.area_score(7.5)
+    assert res.playouts >= 8 * 150
+    assert res.evals + res.cache_hits == res.cache_lookups
+    assert res.sched.requests + res.sched.halted == res.evals   # answered or released, never lost
+    assert res.sched.requests <= res.evals
+    assert 0 < res.sched.requests <= res.sched.batch_slots
+    assert 2 <= res.sched.max_batch_seen <= 8
+    assert res.seconds > 0 and res.visits_per_s > 0
+    print("selfplay: %.0f visits/s, fill %.2f, evals %d, cache hits %d, halted %d, wasted %d" % (
+        res.visits_per_s, res.sched.requests / res.sched.batch_slots, res.evals, res.cache_hits,
+        res.halted, res.wasted), flush=True)
+    # the backend still answers after the last halt/resume
+    pol, val = pipe.forward(netgen.synthetic_inputs(1, seed=1)[0])
+    assert np.isfinite(pol).all() and np.isfinite(val).all()
+    # one thread, same seed: the same game (no scheduling nondeterminism left)
+    cfg1 = pkg.SearchConfig.default(threads=1, visits=60, moves=4, seed=5)
+    r1, m1 = pipe.selfplay(h, cfg1)
+    r2, m2 = pipe.selfplay(h, cfg1)
+    assert m1 == m2 and r1.playouts == r2.playouts
+    pipe.close()
+
+
+def test_selfplay_argument_checks(pkg, netgen, orc):
+    print("case: selfplay argument checks", flush=True)
+    pipe, h, ref, h_ref = make(pkg, netgen, orc, 1, 64, 2, 0, 2)
+    with pytest.raises(ValueError):
+        pipe.selfplay(h, pkg.SearchConfig.default(threads=0))
+    with pytest.raises(ValueError):
+        pipe.selfplay(h, pkg.SearchConfig.default(visits=0))
+    with pytest.raises(ValueError):
+        pipe.get_output(h, np.full((1, 361), 2, np.uint8), 0, symmetry=9)
+    pipe.close()
