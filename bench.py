@@ -73,6 +73,30 @@ def cpu_baseline(orc, netgen, net, x, seconds_budget=20.0):
     }, (pol, val)
 
 
+def calibrate_heads(pipe, netgen, h, batch):
+    """A deep random-init tower feeds the heads planes of magnitude 1e2..1e4, so the
+    softmax is one-hot and tanh saturated: every simulation would follow one line and
+    the search would degenerate.  The fully connected head weights are rescaled (one
+    scalar each, measured on a batch of synthetic positions) so that the policy logits
+    have unit spread and the value pre-activation is centred with spread 0.5 -- the
+    tower, and therefore the device work per evaluation, is unchanged."""
+    import copy
+    x = netgen.synthetic_inputs(min(batch, 32), seed=77)
+    pol, val = pipe.forward_batch(x)
+    relu = lambda a: np.maximum(a, 0.0)
+    p = relu((pol.reshape(-1, 2, 361) - h.bn_pol_mean[None, :, None]) * h.bn_pol_scale[None, :, None])
+    logits = p.reshape(-1, 722) @ h.ip_pol_w.T + h.ip_pol_b
+    v = relu((val - h.bn_val_mean[0]) * h.bn_val_scale[0])
+    hid = relu(v @ h.ip1_val_w.T + h.ip1_val_b)
+    out = hid @ h.ip2_val_w
+    h2 = copy.copy(h)
+    h2.ip_pol_w = (h.ip_pol_w / max(float(logits.std()), 1e-6)).astype(np.float32)
+    g = 0.5 / max(float(out.std()), 1e-6)
+    h2.ip2_val_w = (h.ip2_val_w * g).astype(np.float32)
+    h2.ip2_val_b = np.array([-float(out.mean()) * g], np.float32)
+    return h2
+
+
 def search_workload(args, pkg, netgen):
     """BASELINE configs[4]: tree search with `threads` search threads driving the
     scheduler at max batch `batch`; every move `visits` root visits, `moves` moves of
@@ -84,6 +108,7 @@ def search_workload(args, pkg, netgen):
     pipe = pkg.HIPScheduler(prec, B, device=0)
     pipe.initialize(F)
     pipe.push_weights(6, 18, F, w)
+    h = calibrate_heads(pipe, netgen, h, B)
     cfg = pkg.SearchConfig.default(threads=args.threads, visits=args.visits, moves=args.moves,
                                    seed=2027, reuse_tree=0 if args.no_tree_reuse else 1)
     warm = pkg.SearchConfig.default(threads=args.threads, visits=min(200, args.visits), moves=1,
@@ -99,7 +124,8 @@ def search_workload(args, pkg, netgen):
         "warmup": 1, "ms_per_step": res.seconds / max(1, res.moves_played) * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 storage, f32 accumulate" if prec == pkg.FP16 else "f32",
-        "data": "synthetic (seeded random weights, self-play from the empty board)",
+        "data": "synthetic (seeded random weights, FC head weights rescaled to unsaturated "
+                "outputs, self-play from the empty board)",
         "config": {"workload": "%d search threads, max batch %d, %dx%d %s, %d visits/move, "
                                "%d moves" % (args.threads, B, blocks, F, args.precision,
                                              args.visits, res.moves_played)},
@@ -131,6 +157,9 @@ def main():
     ap.add_argument("--visits", type=int, default=1600)
     ap.add_argument("--moves", type=int, default=20)
     ap.add_argument("--no-tree-reuse", action="store_true")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="only run a plain device copy kernel of MIB mebibytes three times "
+                         "(known traffic, for scaling the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (one replica per GPU, no "
@@ -143,6 +172,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
+    if args.copy_probe:
+        n = args.copy_probe * (1 << 20) // 4
+        a = torch.ones(n, device="cuda")
+        b = torch.empty(n, device="cuda")
+        for _ in range(3):
+            torch.mul(a, 1.0, out=b)      # reads n*4 bytes, writes n*4 bytes
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_mib": args.copy_probe, "bytes_read": n * 4,
+                          "bytes_written": n * 4, "launches": 3}))
+        return
     if args.batch is None:
         args.batch = 64 if args.workload == "forward" else 32
     if args.workload == "search":

@@ -72,6 +72,9 @@ class BatchExecutor {
 public:
     virtual ~BatchExecutor() = default;
     virtual int max_batch() const = 0;
+    // How many forward_batch calls may run at the same time (the scheduler
+    // starts that many worker threads, at most two).
+    virtual int max_concurrency() const { return 1; }
     // in [n][18*361] -> pol [n][722], val [n][361]; throws std::runtime_error.
     virtual void forward_batch(int n, const float* in, float* pol, float* val) = 0;
 };
@@ -92,6 +95,10 @@ std::unique_ptr<BatchExecutor> make_hip_pipe(int device, int precision, int max_
 //  * the worker launches whatever is queued, up to max_batch, after a short
 //    adaptive grace period, instead of "full batch or exactly one"
 //    (.cpp:311-353), so that fewer search threads than max_batch still batch.
+//    The batch it waits for is the number of callers seen around the previous
+//    batches (capped at max_batch); the grace period is bounded by half the
+//    measured execution time of a batch, because at these sizes a forward
+//    costs about the same for 8 positions as for 32.
 class HIPScheduler : public ForwardPipe {
 public:
     // The engine-facing constructor: device pipe created in initialize().
@@ -116,7 +123,8 @@ public:
     lzhip_stats stats();
     void reset_stats();
     // Upper bound, in microseconds, of the grace period the worker grants a
-    // partial batch (0 = launch immediately).
+    // partial batch: 0 = launch immediately, negative = automatic (half the
+    // measured execution time of a batch; the default).
     void set_max_wait_us(int us);
 
 private:
@@ -136,12 +144,15 @@ private:
     std::mutex m_mutex;
     std::condition_variable m_cv;
     std::deque<std::shared_ptr<Request>> m_queue;
-    std::thread m_worker;
+    std::vector<std::thread> m_workers;
+    bool m_collecting = false;  // one worker at a time assembles a batch
     bool m_running = false;
     std::atomic<bool> m_draining{false};
     std::atomic<int> m_outstanding{0};  // callers currently inside forward()
-    int m_max_wait_us = 200;
-    int m_wait_us = 100;
+    int m_max_wait_us = -1;   // < 0: automatic
+    int m_population = 1;     // callers seen around recent batches
+    int m_inflight = 0;       // positions in batches being executed
+    double m_exec_us = 0.0;   // smoothed execution time of a batch
     std::string* m_fail_msg = nullptr;
     // statistics
     std::atomic<uint64_t> m_requests{0}, m_batches{0}, m_halted{0};

@@ -7,6 +7,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <condition_variable>
 #include <cstring>
 #include <map>
 #include <tuple>
@@ -93,9 +94,15 @@ public:
         m_din.alloc(B * kInPlanes * kPts);
         m_dpol.alloc(B * 2 * kPts);
         m_dval.alloc(B * kPts);
-        m_hin.alloc(B * kInPlanes * kPts);
-        m_hpol.alloc(B * 2 * kPts);
-        m_hval.alloc(B * kPts);
+        for (auto& sl : m_slot) {
+            sl.hin.alloc(B * kInPlanes * kPts);
+            sl.hpol.alloc(B * 2 * kPts);
+            sl.hval.alloc(B * kPts);
+            sl.din.alloc(B * kInPlanes * kPts);
+            sl.dpol.alloc(B * 2 * kPts);
+            sl.dval.alloc(B * kPts);
+            HIP_CHECK(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
+        }
         m_act0.alloc(B * kPts * m_C0p);
         for (auto& a : m_act) a.alloc(B * kPts * m_Fp);
         m_V.alloc((size_t)kPos * m_Tp * m_Fp);
@@ -115,10 +122,13 @@ public:
             if (m_ev_start[i]) (void)hipEventDestroy(m_ev_start[i]);
             if (m_ev_stop[i]) (void)hipEventDestroy(m_ev_stop[i]);
         }
+        for (auto& sl : m_slot)
+            if (sl.done) (void)hipEventDestroy(sl.done);
         if (m_stream) (void)hipStreamDestroy(m_stream);
     }
 
     int max_batch() const override { return m_max_batch; }
+    int max_concurrency() const override { return kIoSlots; }
     int filters() const override { return m_filters; }
     int precision() const override { return precision_of<P>(); }
     void* stream() override { return m_stream; }
@@ -185,22 +195,53 @@ public:
         HIP_CHECK(hipStreamSynchronize(m_stream));
     }
 
+    // Host-buffer forward.  Up to kIoSlots callers may be inside at once: each
+    // copies into its own pinned staging, enqueues copy-in, forward and copy-out
+    // on the stream under the pipe lock, and waits for its own event outside
+    // the lock, so that the next batch is queued on the device while this one
+    // runs and host-side copies overlap device work.
     void forward_batch(int n, const float* in, float* pol, float* val) override {
-        std::lock_guard<std::mutex> lk(m_mu);
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
-        std::memcpy(m_hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
-        HIP_CHECK(hipMemcpyAsync(m_din.p, m_hin.p, sizeof(float) * (size_t)n * kInPlanes * kPts,
-                                 hipMemcpyHostToDevice, m_stream));
-        run_forward(n, m_din.p, m_dpol.p, m_dval.p);
-        HIP_CHECK(hipGetLastError());
-        HIP_CHECK(hipMemcpyAsync(m_hpol.p, m_dpol.p, sizeof(float) * (size_t)n * 2 * kPts,
-                                 hipMemcpyDeviceToHost, m_stream));
-        HIP_CHECK(hipMemcpyAsync(m_hval.p, m_dval.p, sizeof(float) * (size_t)n * kPts,
-                                 hipMemcpyDeviceToHost, m_stream));
-        HIP_CHECK(hipStreamSynchronize(m_stream));
-        std::memcpy(pol, m_hpol.p, sizeof(float) * (size_t)n * 2 * kPts);
-        std::memcpy(val, m_hval.p, sizeof(float) * (size_t)n * kPts);
+        IoSlot* sl = nullptr;
+        {
+            std::unique_lock<std::mutex> lk(m_slot_mu);
+            m_slot_cv.wait(lk, [&] {
+                for (auto& c : m_slot)
+                    if (!c.busy) return true;
+                return false;
+            });
+            for (auto& c : m_slot)
+                if (!c.busy) { sl = &c; break; }
+            sl->busy = true;
+        }
+        struct Release {
+            HIPPipeImpl* self;
+            IoSlot* sl;
+            ~Release() {
+                {
+                    std::lock_guard<std::mutex> lk(self->m_slot_mu);
+                    sl->busy = false;
+                }
+                self->m_slot_cv.notify_one();
+            }
+        } release{this, sl};
+        std::memcpy(sl->hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
+        {
+            std::lock_guard<std::mutex> lk(m_mu);
+            HIP_CHECK(hipMemcpyAsync(sl->din.p, sl->hin.p, sizeof(float) * (size_t)n * kInPlanes * kPts,
+                                     hipMemcpyHostToDevice, m_stream));
+            run_forward(n, sl->din.p, sl->dpol.p, sl->dval.p);
+            HIP_CHECK(hipGetLastError());
+            HIP_CHECK(hipMemcpyAsync(sl->hpol.p, sl->dpol.p, sizeof(float) * (size_t)n * 2 * kPts,
+                                     hipMemcpyDeviceToHost, m_stream));
+            HIP_CHECK(hipMemcpyAsync(sl->hval.p, sl->dval.p, sizeof(float) * (size_t)n * kPts,
+                                     hipMemcpyDeviceToHost, m_stream));
+            HIP_CHECK(hipEventRecord(sl->done, m_stream));
+        }
+        HIP_CHECK(hipEventSynchronize(sl->done));
+        std::memcpy(pol, sl->hpol.p, sizeof(float) * (size_t)n * 2 * kPts);
+        std::memcpy(val, sl->hval.p, sizeof(float) * (size_t)n * kPts);
     }
 
     // -------------------------------------------------------------------
@@ -539,8 +580,19 @@ private:
     int m_Fp = 0, m_C0p = 0, m_Tp = 0;
     hipStream_t m_stream = nullptr;
     std::mutex m_mu;
-    DevBuf<float> m_din, m_dpol, m_dval, m_w3, m_scalar;
-    PinnedBuf<float> m_hin, m_hpol, m_hval;
+    DevBuf<float> m_din, m_dpol, m_dval, m_w3, m_scalar;  // evaluate_batch / calibration
+    // Staging of forward_batch: kIoSlots batches may be between "copied in" and
+    // "copied out" at once; their device work is ordered by the one stream.
+    struct IoSlot {
+        PinnedBuf<float> hin, hpol, hval;
+        DevBuf<float> din, dpol, dval;
+        hipEvent_t done = nullptr;
+        bool busy = false;
+    };
+    static constexpr int kIoSlots = 2;
+    IoSlot m_slot[kIoSlots];
+    std::mutex m_slot_mu;
+    std::condition_variable m_slot_cv;
     DevBuf<P> m_act0, m_act[3], m_V, m_M;
     std::vector<Layer> m_layers;
     std::vector<float> m_s;  // activation scales, m_s[0] = input

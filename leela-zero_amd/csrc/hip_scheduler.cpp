@@ -37,7 +37,8 @@ HIPScheduler::~HIPScheduler() {
         m_running = false;
     }
     m_cv.notify_all();
-    if (m_worker.joinable()) m_worker.join();
+    for (auto& w : m_workers)
+        if (w.joinable()) w.join();
     // Anything still queued is released as halted.
     std::deque<std::shared_ptr<Request>> rest;
     {
@@ -58,7 +59,11 @@ void HIPScheduler::start_worker() {
     std::lock_guard<std::mutex> lk(m_mutex);
     if (m_running) return;
     m_running = true;
-    m_worker = std::thread(&HIPScheduler::worker, this);
+    // Two workers when the executor can hold two batches: one assembles and
+    // submits the next batch while the other waits for the device and hands
+    // results back.
+    const int n = std::max(1, std::min(2, m_exec->max_concurrency()));
+    for (int i = 0; i < n; i++) m_workers.emplace_back(&HIPScheduler::worker, this);
 }
 
 // ForwardPipe::initialize (reference src/OpenCLScheduler.cpp:108-132): create
@@ -134,7 +139,7 @@ int HIPScheduler::forward_raw(const float* in, float* pol, float* val) {
         }
         m_queue.push_back(req);
     }
-    m_cv.notify_one();
+    m_cv.notify_all();  // the collecting worker and an idle one share this condition
     int state;
     {
         std::unique_lock<std::mutex> lk(req->mu);
@@ -159,11 +164,15 @@ int HIPScheduler::forward_raw(const float* in, float* pol, float* val) {
 }
 
 // Batch pickup.  The worker sleeps until a request exists, then grants a
-// short grace period for the batch to grow towards the number of callers
-// that are currently inside forward() (they cannot all be queued yet when the
-// first one arrives).  The grace period adapts: it shrinks when it expired
-// without the batch growing and grows, up to m_max_wait_us, when requests
-// kept arriving during it.
+// grace period for the batch to grow towards the number of callers seen around
+// the previous batches (those that were queued or in flight when a batch
+// finished: the threads just answered come back after their host-side work).
+// A forward of a few positions costs about as much as one of a full batch, so
+// waiting a fraction of a batch time for the stragglers beats launching two
+// alternating half batches.  The grace period is bounded by half the measured
+// execution time of a batch (or the fixed value set_max_wait_us gave); an
+// estimate of the callers that is too high costs at most that much per batch
+// and decays by one caller per batch.
 void HIPScheduler::worker() {
     std::vector<float> in, pol, val;
     in.resize((size_t)m_max_batch * kInSize);
@@ -174,41 +183,63 @@ void HIPScheduler::worker() {
         batch.clear();
         {
             std::unique_lock<std::mutex> lk(m_mutex);
-            m_cv.wait(lk, [&] { return !m_running || !m_queue.empty(); });
+            m_cv.wait(lk, [&] { return !m_running || (!m_collecting && !m_queue.empty()); });
             if (!m_running) return;
-            const auto want = [&]() -> size_t {
-                const int o = m_outstanding.load();
-                return (size_t)std::max(1, std::min(m_max_batch, o));
-            };
-            if (m_queue.size() < want() && m_max_wait_us > 0) {
-                const size_t before = m_queue.size();
+            // Only one worker assembles a batch at a time; it hands the role on
+            // when it leaves this block.
+            m_collecting = true;
+            struct Handover {
+                HIPScheduler* s;
+                ~Handover() {
+                    s->m_collecting = false;
+                    s->m_cv.notify_all();
+                }
+            } handover{this};
+            const int cap_us = m_max_wait_us >= 0
+                                   ? m_max_wait_us
+                                   : std::max(50, std::min(5000, (int)(m_exec_us * 0.5)));
+            // Callers known to exist: those seen around recent batches, or inside
+            // forward() right now.  If they all fit one batch, a second batch next
+            // to the one in flight would only split them into two small ones that
+            // cost a full forward each: wait for the device first.  Otherwise the
+            // callers not in flight are the ones this batch can hope for.
+            const int pop = std::max(m_population, m_outstanding.load());
+            size_t target;
+            if (pop <= m_max_batch) {
+                target = (size_t)std::max(1, pop);
+                if (cap_us > 0)
+                    m_cv.wait(lk, [&] {
+                        return !m_running || m_queue.empty() || m_inflight == 0 ||
+                               m_queue.size() >= target;
+                    });
+                if (!m_running) return;
+            } else {
+                target = (size_t)std::max(1, std::min(m_max_batch, pop - m_inflight));
+            }
+            if (m_queue.size() < target && cap_us > 0) {
                 // system_clock: waits on it map to pthread_cond_timedwait, which thread
                 // sanitizers model; the grace period is far too short for clock steps
                 // to matter.
                 const auto deadline =
-                    std::chrono::system_clock::now() + std::chrono::microseconds(m_wait_us);
+                    std::chrono::system_clock::now() + std::chrono::microseconds(cap_us);
                 m_cv.wait_until(lk, deadline, [&] {
-                    return !m_running || m_queue.empty() || m_queue.size() >= want();
+                    return !m_running || m_queue.empty() || m_queue.size() >= target;
                 });
                 if (!m_running) return;
-                if (m_queue.size() < want()) {
-                    if (m_queue.size() > before)
-                        m_wait_us = std::min(m_max_wait_us, m_wait_us * 2 + 1);
-                    else
-                        m_wait_us = std::max(1, m_wait_us / 2);
-                }
             }
             // drain() may have emptied the queue while we waited
             while (!m_queue.empty() && (int)batch.size() < m_max_batch) {
                 batch.push_back(std::move(m_queue.front()));
                 m_queue.pop_front();
             }
+            m_inflight += (int)batch.size();
         }
         if (batch.empty()) continue;
-        const int n = (int)batch.size();
+        const int n = (int)batch.size();  // m_inflight was raised under the lock above
         for (int i = 0; i < n; i++)
             std::memcpy(in.data() + (size_t)i * kInSize, batch[i]->in, sizeof(float) * kInSize);
         int outcome = 1;
+        const auto t0 = std::chrono::steady_clock::now();
         try {
             m_exec->forward_batch(n, in.data(), pol.data(), val.data());
         } catch (const std::exception& e) {
@@ -217,6 +248,16 @@ void HIPScheduler::worker() {
             delete m_fail_msg;
             m_fail_msg = new std::string(e.what());
         }
+        {
+            const double us =
+                std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+            std::lock_guard<std::mutex> lk(m_mutex);
+            m_exec_us = m_exec_us > 0.0 ? 0.75 * m_exec_us + 0.25 * us : us;
+            // callers in flight plus those that queued up meanwhile; forgets slowly
+            m_population = std::max(m_outstanding.load(), m_population - 1);
+            m_inflight -= n;
+        }
+        m_cv.notify_all();  // a collector may be waiting for the device to come free
         m_batches++;
         uint32_t seen = m_max_seen.load();
         while ((uint32_t)n > seen && !m_max_seen.compare_exchange_weak(seen, (uint32_t)n)) {}
@@ -267,8 +308,7 @@ void HIPScheduler::resume() {
 
 void HIPScheduler::set_max_wait_us(int us) {
     std::lock_guard<std::mutex> lk(m_mutex);
-    m_max_wait_us = std::max(0, us);
-    m_wait_us = std::max(1, std::min(m_wait_us, std::max(1, m_max_wait_us)));
+    m_max_wait_us = us < 0 ? -1 : us;
 }
 
 lzhip_stats HIPScheduler::stats() {

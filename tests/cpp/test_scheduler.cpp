@@ -6,7 +6,11 @@
 //   * drain() releases every waiter with a halt, later calls halt at once,
 //     resume() needs an empty queue and re-opens the pipe;
 //   * destruction with idle and with blocked callers ends cleanly;
-//   * an executor failure reaches the caller as an exception.
+//   * an executor failure reaches the caller as an exception;
+//   * with an executor that accepts two batches at a time, two batches are in
+//     flight together and all of the above still holds;
+//   * a steady population of callers smaller than max_batch ends up in one
+//     batch per round instead of two alternating partial ones.
 #include <atomic>
 #include <chrono>
 #include <cstdio>
@@ -37,9 +41,20 @@ std::unique_ptr<BatchExecutor> make_hip_pipe(int, int, int, int) {
 // pol[i] = in[0] + i, val[i] = in[1] - i : each answer identifies its own request.
 class FakeExec : public BatchExecutor {
 public:
-    FakeExec(int mb, int delay_us) : m_mb(mb), m_delay(delay_us) {}
+    FakeExec(int mb, int delay_us, int concurrency = 1)
+        : m_mb(mb), m_delay(delay_us), m_conc(concurrency) {}
     int max_batch() const override { return m_mb; }
+    int max_concurrency() const override { return m_conc; }
     void forward_batch(int n, const float* in, float* pol, float* val) override {
+        struct InFlight {
+            FakeExec* e;
+            explicit InFlight(FakeExec* x) : e(x) {
+                const int now = ++e->inside;
+                int seen = e->max_inside.load();
+                while (now > seen && !e->max_inside.compare_exchange_weak(seen, now)) {}
+            }
+            ~InFlight() { --e->inside; }
+        } in_flight(this);
         if (n < 1 || n > m_mb) { oversize = true; }
         if (fail_next.exchange(false)) throw std::runtime_error("injected failure");
         std::this_thread::sleep_for(std::chrono::microseconds(m_delay));
@@ -52,9 +67,9 @@ public:
         positions += n;
     }
     std::atomic<bool> oversize{false}, fail_next{false};
-    std::atomic<int> calls{0}, positions{0};
+    std::atomic<int> calls{0}, positions{0}, inside{0}, max_inside{0};
 private:
-    int m_mb, m_delay;
+    int m_mb, m_delay, m_conc;
 };
 
 static void one_call(HIPScheduler& s, float a, float b, std::atomic<int>& ok,
@@ -72,8 +87,8 @@ static void one_call(HIPScheduler& s, float a, float b, std::atomic<int>& ok,
     }
 }
 
-static void test_concurrent(int threads, int mb, int reps) {
-    auto* fe = new FakeExec(mb, 200);
+static void test_concurrent(int threads, int mb, int reps, int concurrency = 1) {
+    auto* fe = new FakeExec(mb, 200, concurrency);
     HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
     std::atomic<int> ok{0}, halted{0};
     std::vector<std::thread> th;
@@ -90,9 +105,36 @@ static void test_concurrent(int threads, int mb, int reps) {
     CHECK(st.max_batch_seen <= (uint32_t)mb);
     CHECK(st.batches == (uint64_t)fe->calls.load());
     if (threads >= 2 * mb) CHECK(st.batches < (uint64_t)threads * reps);  // it did batch
+    CHECK(fe->max_inside <= concurrency);
+    if (concurrency == 2 && threads >= 4 * mb) CHECK(fe->max_inside == 2);  // batches overlapped
     std::printf("concurrent threads=%d mb=%d: %llu batches for %llu requests, max %u\n", threads,
                 mb, (unsigned long long)st.batches, (unsigned long long)st.requests,
                 st.max_batch_seen);
+}
+
+// 12 callers that come straight back after each answer, max batch 32: once the
+// scheduler has seen the population it waits for all of them, so the mean
+// batch approaches 12 instead of the 6+6 of two alternating groups.
+static void test_population_batches(int concurrency) {
+    auto* fe = new FakeExec(32, 2000, concurrency);
+    HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
+    std::atomic<int> ok{0}, halted{0};
+    std::vector<std::thread> th;
+    const int threads = 12, reps = 40;
+    for (int t = 0; t < threads; t++)
+        th.emplace_back([&, t] {
+            for (int r = 0; r < reps; r++) {
+                one_call(s, (float)t, (float)r, ok, halted);
+                std::this_thread::sleep_for(std::chrono::microseconds(100 + 20 * t));  // host work
+            }
+        });
+    for (auto& t : th) t.join();
+    const lzhip_stats st = s.stats();
+    CHECK(ok == threads * reps);
+    const double mean = (double)st.requests / (double)st.batches;
+    std::printf("population (executor concurrency %d): %llu batches, mean batch %.1f of %d callers\n",
+                concurrency, (unsigned long long)st.batches, mean, threads);
+    CHECK(mean >= 9.0);
 }
 
 static void test_drain_resume() {
@@ -165,6 +207,10 @@ int main() {
     test_concurrent(1, 4, 20);
     test_concurrent(16, 32, 30);   // fewer callers than max_batch: must still batch, never stall
     test_concurrent(48, 8, 20);
+    test_concurrent(48, 8, 20, 2);  // two batches in flight
+    test_concurrent(5, 8, 20, 2);
+    test_population_batches(1);
+    test_population_batches(2);
     test_drain_resume();
     test_destroy_with_waiters();
     test_executor_failure();
