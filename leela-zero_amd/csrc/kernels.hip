@@ -928,8 +928,8 @@ __global__ __launch_bounds__(256, 2) void wino_gemm_persistent_k(
 template <typename P, int NK>
 __global__ __launch_bounds__(512) void wino_gemm_big_k(const P* __restrict__ V,
                                                        const P* __restrict__ U,
-                                                       P* __restrict__ M, int Tp, int Cp, int Kp,
-                                                       int tiles_m, int tiles_n, int seg) {
+                                                       P* __restrict__ M, int T, int Tp, int Cp,
+                                                       int Kp, int tiles_m, int tiles_n, int seg) {
     constexpr int BM = 256, BN = 256, NT = 512;
     constexpr int EPC = 16 / sizeof(P);
     constexpr int BK = 128 / sizeof(P);
@@ -957,7 +957,13 @@ __global__ __launch_bounds__(512) void wino_gemm_big_k(const P* __restrict__ V,
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wy = wave >> 2, wx = wave & 3;
     const int lrow = tid >> 3, lch = tid & 7;   // 64 rows per pass of the workgroup
-    const P* Ag = V + ((size_t)p * Tp + (size_t)tm * BM + lrow) * Cp + lch * EPC;
+    // Rows past the last real tile re-read row T-1 (their products are never stored).
+    const P* Ag[A_CH];
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) {
+        const int row = min(tm * BM + lrow + i * 64, T - 1);
+        Ag[i] = V + ((size_t)p * Tp + row) * Cp + lch * EPC;
+    }
     const P* Bg = U + ((size_t)p * Kp + (size_t)tn * BN + lrow) * Cp + lch * EPC;
 
     float16v acc[MB][NB];
@@ -972,7 +978,7 @@ __global__ __launch_bounds__(512) void wino_gemm_big_k(const P* __restrict__ V,
     auto gload = [&](int st, int k0) {
 #pragma unroll
         for (int i = 0; i < A_CH; i++)
-            ra[st][i] = *reinterpret_cast<const int4v*>(Ag + (size_t)(i * 64) * Cp + k0);
+            ra[st][i] = *reinterpret_cast<const int4v*>(Ag[i] + k0);
 #pragma unroll
         for (int i = 0; i < B_CH; i++)
             rb[st][i] = *reinterpret_cast<const int4v*>(Bg + (size_t)(i * 64) * Cp + k0);
@@ -1028,6 +1034,7 @@ __global__ __launch_bounds__(512) void wino_gemm_big_k(const P* __restrict__ V,
     const int ccol = 4 * (lane >> 5), crow = lane & 31;
     constexpr int CPR = BN / EPC;
     P* Mg = M + ((size_t)p * Tp + (size_t)tm * BM) * Kp + (size_t)tn * BN;
+    const int real_rows = T - tm * BM;   // rows of this tile that hold tiles of a board
 #pragma unroll
     for (int part = 0; part < EP_PARTS; part++) {
 #pragma unroll
@@ -1051,8 +1058,9 @@ __global__ __launch_bounds__(512) void wino_gemm_big_k(const P* __restrict__ V,
 #pragma unroll 4
         for (int q = tid; q < PROWS * CPR; q += NT) {
             const int row = q / CPR, ch = q - row * CPR;
-            *reinterpret_cast<int4v*>(Mg + (size_t)(part * PROWS + row) * Kp + ch * EPC) =
-                *reinterpret_cast<const int4v*>(&smem[row * CROW + ch * EPC]);
+            if (part * PROWS + row < real_rows)   // padding rows are never read back
+                *reinterpret_cast<int4v*>(Mg + (size_t)(part * PROWS + row) * Kp + ch * EPC) =
+                    *reinterpret_cast<const int4v*>(&smem[row * CROW + ch * EPC]);
         }
         __syncthreads();
     }
@@ -1093,14 +1101,14 @@ static void launch_gemm_bn(const P* V, const P* U, P* M, int tiles_m, int Tp, in
 }
 
 template <typename P, int NK>
-static void launch_gemm_big(const P* V, const P* U, P* M, int tiles_m, int Tp, int Cp, int Kp,
-                            hipStream_t s, LaunchTimer* t) {
+static void launch_gemm_big(const P* V, const P* U, P* M, int T, int tiles_m, int Tp, int Cp,
+                            int Kp, hipStream_t s, LaunchTimer* t) {
     const int tiles_n = Kp / 256;
     const int n_items = kPos * tiles_m * tiles_n;
     int seg = (n_items + 7) / 8;
     seg = (seg + tiles_n - 1) / tiles_n * tiles_n;
-    launch(wino_gemm_big_k<P, NK>, dim3(8 * seg), dim3(512), s, t, V, U, M, Tp, Cp, Kp, tiles_m,
-           tiles_n, seg);
+    launch(wino_gemm_big_k<P, NK>, dim3(8 * seg), dim3(512), s, t, V, U, M, T, Tp, Cp, Kp,
+           tiles_m, tiles_n, seg);
 }
 
 // T = number of real tile rows (25 per board); Tp (the row count of V and M)
@@ -1114,7 +1122,7 @@ void launch_gemm(const P* V, const P* U, P* M, int T, int Tp, int Cp, int Kp, hi
     const int big_rows = (T + 255) / 256;
     if (Kp % 256 == 0 && big_rows * (Kp / 256) * kPos >= 160) {
         switch (nk) {
-#define LZ_BIG(N) case N: launch_gemm_big<P, N>(V, U, M, big_rows, Tp, Cp, Kp, s, t); return;
+#define LZ_BIG(N) case N: launch_gemm_big<P, N>(V, U, M, T, big_rows, Tp, Cp, Kp, s, t); return;
             LZ_BIG(1) LZ_BIG(2) LZ_BIG(4) LZ_BIG(8) LZ_BIG(16)
 #undef LZ_BIG
             default: break;
