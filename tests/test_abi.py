@@ -94,3 +94,32 @@ def test_weights_file_round_trip(netgen, tmp_path):
     (tmp_path / "short.txt").write_text("\n".join(lines[:-3]) + "\n")
     with pytest.raises(ValueError):
         netgen.load_weights(tmp_path / "short.txt")
+
+
+GOLDEN_NET = os.path.join(ROOT, "tests", "golden", "0k.txt.gz")
+
+
+def test_reference_weights_fixture_loads(netgen, orc, tmp_path):
+    """tests/golden/0k.txt.gz is the weights file the reference's own unit tests load
+    (src/tests/0k.txt, gzip-compressed; the reference reads gzip too): format version 1,
+    one residual block of 8 filters."""
+    net = netgen.load_weights(GOLDEN_NET)
+    assert (net.blocks, net.filters, net.value_head_not_stm) == (1, 8, False)
+    sizes = [np.asarray(v).size for v in net.lines()]
+    assert sizes == [1296, 8, 8, 8, 576, 8, 8, 8, 576, 8, 8, 8,
+                     16, 2, 2, 2, 261364, 362, 8, 1, 1, 1, 92416, 256, 256, 1]
+    # the file survives a write/read cycle of this package's writer
+    out = tmp_path / "again.txt"
+    netgen.save_weights(net, out)
+    back = netgen.load_weights(out)
+    for a, b in zip(net.lines(), back.lines()):
+        assert np.array_equal(np.asarray(a, np.float32).ravel(), np.asarray(b, np.float32).ravel())
+    # and the CPU oracle evaluates it to a proper distribution
+    w, h = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    ref = orc.OraclePipe()
+    ref.initialize(net.filters)
+    ref.push_weights(6, 18, net.filters, w)
+    pol, val = ref.forward(netgen.synthetic_inputs(1, seed=9)[0])
+    hd = orc.heads(h, pol, val)
+    assert abs(float(hd["policy"].sum()) - 1.0) < 1e-5 and 0.0 < hd["winrate"] < 1.0
+    assert hd["policy"].max() < 0.9      # a real network: not a saturated one-hot

@@ -174,6 +174,27 @@ def test_golden_fixtures_on_device(pkg, netgen):
 
 
 @pytest.mark.parametrize("precision", [0, 1])
+def test_reference_weights_file_on_device(pkg, netgen, orc, precision):
+    """The weights file of the reference's own unit tests (1 block x 8 filters, loaded
+    through the text-format reader) against the oracle: 8 filters exercise the padding of
+    the channel dimension to 64 with real weights."""
+    import os
+    print("case: reference weights file precision=%d" % precision, flush=True)
+    net = netgen.load_weights(os.path.join(os.path.dirname(__file__), "golden", "0k.txt.gz"))
+    w, h = netgen.prepare(net)
+    w_ref, h_ref = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    ref = orc.OraclePipe()
+    ref.initialize(net.filters)
+    ref.push_weights(6, 18, net.filters, w_ref)
+    pipe = pkg.HIPScheduler(precision, 8)
+    pipe.initialize(net.filters)
+    pipe.push_weights(6, 18, net.filters, w)
+    pipe.push_heads(h)
+    check_outputs(pkg, orc, pipe, ref, h_ref, netgen.synthetic_inputs(8, seed=31), precision)
+    pipe.close()
+
+
+@pytest.mark.parametrize("precision", [0, 1])
 def test_batch_composition_does_not_change_results(pkg, netgen, orc, precision):
     """A position evaluated alone, in a partial batch and in a full batch gives
     bit-identical planes (rows of the GEMM are independent)."""
