@@ -21,6 +21,13 @@ PEAK_MFMA_F16 = 2.5e15   # dense fp16 matrix FLOP/s, MI355X
 PEAK_MFMA_F32 = 157.3e12
 PEAK_HBM = 8.0e12        # bytes/s
 
+# HBM bytes per launch of the Winograd GEMM, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch, scaled by what the same counters read for a plain copy kernel of known
+# size: x2.0 and x1.0); summary and commands in profiles/gemm_and_transform_40x256_fp16_b64_pmc.txt.
+# Counters cannot be read from inside this process, so the figure is only reported for the
+# workload it was measured on: (blocks, filters, precision, batch).
+MEASURED_GEMM_TRAFFIC = {(40, 256, "fp16", 64): (17172.8 * 2.0 + 28800.0 * 1.0) * 1024.0}
+
 
 def gemm_flops(batch, filters, n_layers):
     """Algorithmic flops of the 36 batched GEMMs of one forward:
@@ -47,7 +54,7 @@ def transform_bytes(batch, filters, n_layers, e):
     return in_t, out_t, fused
 
 
-def cpu_baseline(orc, netgen, net, x, seconds_budget=20.0):
+def cpu_baseline(orc, netgen, net, x, seconds_budget=15.0):
     """CPU oracle timed on this host: independent single-position forwards on all
     the cores this process may use (the shape of the reference's netbench)."""
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
@@ -60,8 +67,7 @@ def cpu_baseline(orc, netgen, net, x, seconds_budget=20.0):
     t0 = time.perf_counter()
     ref.forward(x[0])
     one = time.perf_counter() - t0
-    per_thread = max(1, int(seconds_budget / max(one, 1e-3)))
-    per_thread = min(per_thread, 8)
+    per_thread = max(1, min(256, int(seconds_budget / max(one, 1e-3))))
     n = cores * per_thread
     xs = np.concatenate([x] * (n // x.shape[0] + 1))[:n]
     pol, val, secs = ref.forward_many(xs, threads=cores)
@@ -234,7 +240,9 @@ def main():
     roofline = {
         "kernel": "wino_gemm_k (36-way batched Winograd GEMM)",
         "bound": "mfma", "achieved": gemm_rate / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
-        "frac": gemm_rate / peak, "traffic": None,
+        "frac": gemm_rate / peak,
+        "traffic": MEASURED_GEMM_TRAFFIC.get((blocks, F, args.precision, B)),
+        "algorithmic_bytes_per_launch": 36.0 * e * (25 * B * F * 2 + F * F),
         "avg_launch_us": ms[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],
         "launches_per_forward": int(cnt[pkg.K_GEMM]),
         "flops_per_launch": gf / cnt[pkg.K_GEMM],
