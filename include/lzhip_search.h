@@ -91,6 +91,15 @@ int lzhip_get_output(lzhip_handle* h, const lzhip_head_weights* heads, const uin
                      int n_boards, int to_move, int symmetry, float softmax_temp,
                      float* policy, float* winrate);
 
+/* Network::get_output with Ensemble::AVERAGE (reference src/Network.cpp:762-775):
+ * the mean over the eight symmetries of policy, pass probability and winrate.
+ * The eight symmetric inputs are evaluated as device batches (one batch of 8
+ * when max_batch >= 8) directly on the pipe, not through the request queue, so
+ * drain() does not interrupt it; heads run on the calling thread. */
+int lzhip_get_output_average(lzhip_handle* h, const lzhip_head_weights* heads,
+                             const uint8_t* boards, int n_boards, int to_move,
+                             float softmax_temp, float* policy, float* winrate);
+
 int lzhip_search_default_config(lzhip_search_config* cfg);
 
 /* Self-play from the empty board with cfg->threads search threads calling the

@@ -44,6 +44,7 @@ EXPORTS = [
 # Every symbol include/lzhip_search.h declares.
 SEARCH_EXPORTS = [
     "lzhip_symmetry_index", "lzhip_gather_features", "lzhip_get_output",
+    "lzhip_get_output_average",
     "lzhip_search_default_config", "lzhip_selfplay", "lzhip_board_replay",
 ]
 
@@ -152,6 +153,8 @@ def lib():
         L.lzhip_get_output.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights), _u8p,
                                        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float,
                                        _fp, _fp]
+        L.lzhip_get_output_average.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights), _u8p,
+                                               ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
         L.lzhip_search_default_config.argtypes = [ctypes.POINTER(SearchConfig)]
         L.lzhip_selfplay.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights),
                                      ctypes.POINTER(SearchConfig), ctypes.POINTER(SearchResult),
@@ -423,6 +426,21 @@ class HIPScheduler:
         _check(lib().lzhip_get_output(self._h, ctypes.byref(c), bp, b.shape[0], int(to_move),
                                       int(symmetry), float(temperature), _ptr(policy),
                                       ctypes.byref(win)))
+        del keep
+        return policy, win.value
+
+    def get_output_average(self, heads, boards, to_move, temperature=1.0):
+        """Network::get_output with Ensemble::AVERAGE (reference
+        src/Network.cpp:762-775): mean over the 8 symmetries, evaluated as one
+        device batch.  Returns (policy[362], winrate)."""
+        self._need()
+        c, keep = _c_heads(heads)
+        b, bp = _boards(boards)
+        policy = np.empty(MOVES, dtype=np.float32)
+        win = ctypes.c_float()
+        _check(lib().lzhip_get_output_average(self._h, ctypes.byref(c), bp, b.shape[0],
+                                              int(to_move), float(temperature), _ptr(policy),
+                                              ctypes.byref(win)))
         del keep
         return policy, win.value
 

@@ -1,6 +1,7 @@
 // extern "C" surface declared in include/lzhip.h.  Every function converts
 // C++ exceptions into return codes; the message of the last failure is kept
 // per calling thread.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <memory>
@@ -285,6 +286,44 @@ int lzhip_get_output(lzhip_handle* h, const lzhip_head_weights* heads, const uin
     heads_on_host(hw, pol.data(), val.data(), softmax_temp, p, winrate);
     for (int i = 0; i < go::kPoints; i++) policy[symmetry_index(symmetry, i)] = p[i];
     policy[go::kPoints] = p[go::kPoints];
+    return LZHIP_OK;
+    GUARD_END
+}
+
+int lzhip_get_output_average(lzhip_handle* h, const lzhip_head_weights* heads,
+                             const uint8_t* boards, int n_boards, int to_move,
+                             float softmax_temp, float* policy, float* winrate) {
+    if (!h || !heads_complete(heads) || !boards || !policy || !winrate)
+        return fail(LZHIP_EINVAL, "null argument");
+    if (!(softmax_temp > 0.0f)) return fail(LZHIP_EINVAL, "softmax_temp must be positive");
+    GUARD_BEGIN
+    constexpr int S = 8;
+    std::vector<float> in((size_t)S * LZHIP_INPUT_SIZE), pol((size_t)S * LZHIP_POL_SIZE),
+        val((size_t)S * LZHIP_VAL_SIZE);
+    for (int sym = 0; sym < S; sym++) {
+        const int rc = lzhip_gather_features(boards, n_boards, to_move, sym,
+                                             in.data() + (size_t)sym * LZHIP_INPUT_SIZE);
+        if (rc != LZHIP_OK) return rc;
+    }
+    const int step = std::min(S, h->pipe->max_batch());
+    for (int s0 = 0; s0 < S; s0 += step) {
+        const int n = std::min(step, S - s0);
+        h->pipe->forward_batch(n, in.data() + (size_t)s0 * LZHIP_INPUT_SIZE,
+                               pol.data() + (size_t)s0 * LZHIP_POL_SIZE,
+                               val.data() + (size_t)s0 * LZHIP_VAL_SIZE);
+    }
+    const HeadWeights hw(*heads);
+    for (int i = 0; i <= go::kPoints; i++) policy[i] = 0.0f;
+    float win = 0.0f;
+    for (int sym = 0; sym < S; sym++) {
+        float p[go::kPoints + 1], w;
+        heads_on_host(hw, pol.data() + (size_t)sym * LZHIP_POL_SIZE,
+                      val.data() + (size_t)sym * LZHIP_VAL_SIZE, softmax_temp, p, &w);
+        for (int i = 0; i < go::kPoints; i++) policy[symmetry_index(sym, i)] += p[i] / (float)S;
+        policy[go::kPoints] += p[go::kPoints] / (float)S;
+        win += w / (float)S;
+    }
+    *winrate = win;
     return LZHIP_OK;
     GUARD_END
 }

@@ -53,6 +53,17 @@ uint64_t Position::hash() const {
     return h;
 }
 
+uint64_t Position::mapped_hash(const int16_t* map) const {
+    const Tables& t = tables();
+    uint64_t h = 0;
+    for (int v = 0; v < kPoints; v++)
+        if (m_sq[v] != EMPTY) h ^= t.zob[m_sq[v]][map[v]];
+    if (m_to_move == WHITE) h ^= t.zob_white_to_move;
+    h ^= t.zob_ko[m_ko < 0 ? kPoints : map[m_ko]];
+    h ^= t.zob_pass[std::min(m_passes, 3)];
+    return h;
+}
+
 void Position::analyze(GroupInfo& g) const {
     const Tables& t = tables();
     std::memset(g.id, 0xff, sizeof(g.id));

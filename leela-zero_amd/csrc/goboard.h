@@ -63,6 +63,9 @@ public:
     // (the reference's FastBoard hash covers the same state).
     uint64_t hash() const;
     uint64_t stone_hash() const { return m_stone_hash; }
+    // hash() of the position in which every point v has moved to map[v]
+    // (reference FullBoard::calc_symmetry_hash, src/FullBoard.cpp:111-122).
+    uint64_t mapped_hash(const int16_t* map) const;
 
     void analyze(GroupInfo& g) const;
     // Empty, not the ko point, not suicide (needs analyze() of this position).

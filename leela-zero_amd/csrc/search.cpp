@@ -197,11 +197,34 @@ Netresult NetworkFacade::get_output_internal(const go::Position& pos, int symmet
     return r;
 }
 
+bool NetworkFacade::probe_cache(const go::Position& pos, Netresult& out) {
+    if (m_cache.lookup(pos.hash(), out)) return true;
+    // opening_moves(19) / 2 = (361 / 6) / 2 (reference src/TimeControl.cpp:300-304)
+    if (!m_symmetry_probe || pos.movenum() >= (kPoints / 6) / 2) return false;
+    for (int sym = 1; sym < 8; sym++) {
+        const int16_t* map = sym_table().idx[sym];
+        Netresult cached;
+        if (m_cache.lookup(pos.mapped_hash(map), cached)) {
+            for (int i = 0; i < kPoints; i++) out.policy[i] = cached.policy[map[i]];
+            out.policy_pass = cached.policy_pass;
+            out.winrate = cached.winrate;
+            return true;
+        }
+    }
+    return false;
+}
+
 Netresult NetworkFacade::get_output(const go::Position& pos, int symmetry, uint64_t& rng_state,
                                     bool use_cache) {
     Netresult r;
     const uint64_t key = pos.hash();
-    if (use_cache && m_cache.lookup(key, r)) return r;
+    if (use_cache) {
+        m_probes++;
+        if (probe_cache(pos, r)) {
+            m_probe_hits++;
+            return r;
+        }
+    }
     if (symmetry < 0) symmetry = (int)(next_rand(rng_state) >> 61);
     r = get_output_internal(pos, symmetry);
     if (use_cache) m_cache.insert(key, r);
@@ -568,6 +591,7 @@ void selfplay(ForwardPipe& pipe, const lzhip_head_weights& heads, const lzhip_se
     if (sched) before = sched->stats();
 
     NetworkFacade net(pipe, heads, (size_t)std::max(cfg.cache_size, 0), cfg.softmax_temp);
+    net.set_symmetry_probe(cfg.random_moves == 0);  // as the reference: not in randomised self-play
     UCTSearch search(net, cfg);
     go::Position pos;
     const auto t0 = std::chrono::steady_clock::now();
@@ -586,8 +610,8 @@ void selfplay(ForwardPipe& pipe, const lzhip_head_weights& heads, const lzhip_se
     out.halted = st.halted;
     out.nodes = st.nodes;
     out.evals = net.evals();
-    out.cache_lookups = net.cache().lookups();
-    out.cache_hits = net.cache().hits();
+    out.cache_lookups = net.cache_lookups();
+    out.cache_hits = net.cache_hits();
     out.seconds = std::chrono::duration<double>(t1 - t0).count();
     out.visits_per_s = out.seconds > 0 ? (double)out.playouts / out.seconds : 0.0;
     out.moves_played = played;

@@ -95,17 +95,27 @@ public:
     Netresult get_output(const go::Position& pos, int symmetry, uint64_t& rng_state,
                          bool use_cache = true);
     Netresult get_output_internal(const go::Position& pos, int symmetry);
+    // Cache lookup as Network::probe_cache (reference src/Network.cpp:717-742):
+    // the position itself, then, during the first 30 moves and when enabled,
+    // its seven symmetric images (their cached policy is mapped back).
+    bool probe_cache(const go::Position& pos, Netresult& out);
+    void set_symmetry_probe(bool on) { m_symmetry_probe = on; }
     void drain() { m_pipe.drain(); }
     void resume() { m_pipe.resume(); }
     EvalCache& cache() { return m_cache; }
     uint64_t evals() const { return m_evals.load(); }
+    // get_output calls that consulted the cache, and those it answered
+    // (directly or through a symmetric image).
+    uint64_t cache_lookups() const { return m_probes.load(); }
+    uint64_t cache_hits() const { return m_probe_hits.load(); }
 
 private:
     ForwardPipe& m_pipe;
     HeadWeights m_heads;
     EvalCache m_cache;
     float m_temp;
-    std::atomic<uint64_t> m_evals{0};
+    bool m_symmetry_probe = true;
+    std::atomic<uint64_t> m_evals{0}, m_probes{0}, m_probe_hits{0};
 };
 
 struct SearchStats {

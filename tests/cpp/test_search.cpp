@@ -12,7 +12,9 @@
 //   * requests still queued at the end of a move are released by the halt and
 //     the scheduler answers again afterwards;
 //   * one thread with one seed plays the same game twice;
-//   * the evaluation cache answers repeated positions;
+//   * the evaluation cache answers repeated positions, and in the opening also
+//     the seven symmetric images of a cached position, with the policy mapped
+//     back to the asking position's board order;
 //   * a finished game (two passes) is not searched;
 //   * an executor failure reaches the caller as an exception.
 #include <atomic>
@@ -158,6 +160,41 @@ static void test_unrotation() {
     }
 }
 
+static void test_symmetric_cache_probe() {
+    HIPScheduler sched(std::make_unique<NeighbourNet>(4, 0));
+    Heads heads;
+    NetworkFacade net(sched, heads.c, 100, 1.0f);
+    uint64_t rng = 5;
+    // black (2,5), white (9,3): no symmetry of its own
+    go::Position a;
+    a.play(5 * 19 + 2);
+    a.play(3 * 19 + 9);
+    const Netresult ra = net.get_output(a, 0, rng);
+    CHECK(net.evals() == 1 && net.cache_hits() == 0);
+    for (int sym = 1; sym < 8; sym++) {
+        // the same game seen through symmetry `sym`
+        go::Position b;
+        b.play(symmetry_index(sym, 5 * 19 + 2));
+        b.play(symmetry_index(sym, 3 * 19 + 9));
+        const Netresult direct = net.get_output(b, 0, rng, /*use_cache=*/false);
+        const uint64_t evals_before = net.evals();
+        const Netresult cached = net.get_output(b, 0, rng);
+        CHECK(net.evals() == evals_before);           // answered from a's entry
+        CHECK(net.cache_hits() == (uint64_t)sym);
+        for (int i = 0; i < kPoints; i++) CHECK(std::fabs(cached.policy[i] - direct.policy[i]) < 1e-6f);
+        CHECK(std::fabs(cached.winrate - direct.winrate) < 1e-6f);
+        CHECK(std::fabs(cached.winrate - ra.winrate) < 1e-6f);
+    }
+    // switched off, or after the opening, the images are not consulted
+    net.set_symmetry_probe(false);
+    go::Position c;
+    c.play(symmetry_index(3, 5 * 19 + 2));
+    c.play(symmetry_index(3, 3 * 19 + 9));
+    const uint64_t evals_before = net.evals();
+    net.get_output(c, 0, rng);
+    CHECK(net.evals() == evals_before + 1);
+}
+
 static std::vector<int> play_game(int threads, int visits, int moves, int delay_us, int max_batch,
                                   lzhip_search_result* res_out, int reuse = 1) {
     HIPScheduler sched(std::make_unique<NeighbourNet>(max_batch, delay_us));
@@ -196,8 +233,8 @@ static std::vector<int> play_game(int threads, int visits, int moves, int delay_
         res_out->halted = search.stats().halted;
         res_out->wasted = search.stats().wasted;
         res_out->evals = net.evals();
-        res_out->cache_hits = net.cache().hits();
-        res_out->cache_lookups = net.cache().lookups();
+        res_out->cache_hits = net.cache_hits();
+        res_out->cache_lookups = net.cache_lookups();
         res_out->sched = sched.stats();
     }
     return game;
@@ -295,6 +332,8 @@ static void test_selfplay_entry_and_failure() {
 int main() {
     std::printf("unrotation\n");
     test_unrotation();
+    std::printf("symmetric cache probe\n");
+    test_symmetric_cache_probe();
     std::printf("single thread\n");
     test_single_thread_deterministic();
     std::printf("many threads\n");

@@ -61,6 +61,33 @@ def test_get_output_matches_oracle_chain(pkg, netgen, orc, precision):
     pipe.close()
 
 
+@pytest.mark.parametrize("max_batch", [8, 3])
+def test_average_ensemble_matches_oracle(pkg, netgen, orc, max_batch):
+    """Mean over the 8 symmetries, as one device batch (or chunks when max_batch < 8)."""
+    print("case: average ensemble max_batch=%d" % max_batch, flush=True)
+    pipe, h, ref, h_ref = make(pkg, netgen, orc, 2, 64, 13, 0, max_batch)
+    orc.use_builtin()
+    b, boards = random_position(9, 90)
+    policy, winrate = pipe.get_output_average(h, np.array(boards, np.uint8), b.to_move)
+    want = np.zeros(362, np.float64)
+    want_win = 0.0
+    for sym in range(8):
+        planes = np.array(G.gather_features(boards, b.to_move, sym), np.float32)
+        rp, rv = ref.forward(planes)
+        hd = orc.heads(h_ref, rp, rv)
+        for idx in range(361):
+            want[G.symmetry_index(sym, idx)] += hd["policy"][idx] / 8.0
+        want[361] += hd["policy"][361] / 8.0
+        want_win += hd["winrate"] / 8.0
+    assert float(np.abs(policy - want).max()) <= 1e-4
+    assert abs(winrate - want_win) <= 1e-4
+    assert abs(float(policy.sum()) - 1.0) < 1e-4
+    # the position is not symmetric, so the mean differs from any single symmetry
+    single, _ = pipe.get_output(h, np.array(boards, np.uint8), b.to_move, 0)
+    assert float(np.abs(single - policy).max()) > 1e-4
+    pipe.close()
+
+
 def test_selfplay_on_device(pkg, netgen, orc):
     print("case: selfplay 2x64 fp16, 12 threads, batch 8", flush=True)
     pipe, h, ref, h_ref = make(pkg, netgen, orc, 2, 64, 21, 1, 8)
