@@ -51,7 +51,27 @@ def build(verbose=False):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    build_engine_path_test(verbose)
     return LIB
+
+
+ENGINE_TEST = os.path.join(CSRC, "engine_path_test")
+
+
+def build_engine_path_test(verbose=False):
+    """tests/cpp/test_engine_path.cpp linked against the library: the C++ drop-in
+    path (HIPScheduler as a ForwardPipe) exercised on a GPU box by the GPU tests.
+    Built here so that no compiler has to run there."""
+    src = os.path.join(ROOT, "tests", "cpp", "test_engine_path.cpp")
+    cmd = [hipcc(), "-O1", "-std=c++17", "-x", "c++", src, "-x", "none",
+           "-I", os.path.join(ROOT, "include"), "-L", CSRC, "-llzhip", "-lpthread",
+           "-Wl,-rpath,$ORIGIN", "-o", ENGINE_TEST]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("engine path test failed to build:\n" + r.stderr)
+    return ENGINE_TEST
 
 
 if __name__ == "__main__":
