@@ -20,7 +20,9 @@ extern "C" {
 
 /* Head parameters as Network holds them (reference src/Network.h:166-183)
  * after the preprocessing of src/Network.cpp:351-352,568-576; same meaning as
- * the arguments of lzhip_push_heads. */
+ * the arguments of lzhip_push_heads.  Every entry point below that takes a
+ * `heads` argument accepts NULL for "the parameters given to lzhip_push_heads"
+ * (kept in host layout by the handle, so repeated calls do not re-pack them). */
 typedef struct lzhip_head_weights {
     const float* bn_pol_mean;  /* [2]   conv bias folded in              */
     const float* bn_pol_scale; /* [2]   1/sqrt(var+1e-5)                 */

@@ -237,7 +237,10 @@ def board_replay(moves, komi=7.5):
 
 
 def _c_heads(heads):
-    """(struct, keep-alive arrays) for a HeadWeights-like object."""
+    """(pointer argument, keep-alive objects) for a HeadWeights-like object; None
+    stands for the parameters given to push_heads."""
+    if heads is None:
+        return None, None
     arrs, c = [], CHeadWeights()
     for name, size in zip(HeadWeights.FIELDS, HeadWeights.SIZES):
         a = _f32(getattr(heads, name)).reshape(-1)
@@ -245,7 +248,7 @@ def _c_heads(heads):
             raise ValueError("%s must have %d values" % (name, size))
         arrs.append(a)
         setattr(c, name, _ptr(a))
-    return c, arrs
+    return ctypes.byref(c), (c, arrs)
 
 
 class ForwardPipeWeights:
@@ -423,7 +426,7 @@ class HIPScheduler:
         b, bp = _boards(boards)
         policy = np.empty(MOVES, dtype=np.float32)
         win = ctypes.c_float()
-        _check(lib().lzhip_get_output(self._h, ctypes.byref(c), bp, b.shape[0], int(to_move),
+        _check(lib().lzhip_get_output(self._h, c, bp, b.shape[0], int(to_move),
                                       int(symmetry), float(temperature), _ptr(policy),
                                       ctypes.byref(win)))
         del keep
@@ -438,7 +441,7 @@ class HIPScheduler:
         b, bp = _boards(boards)
         policy = np.empty(MOVES, dtype=np.float32)
         win = ctypes.c_float()
-        _check(lib().lzhip_get_output_average(self._h, ctypes.byref(c), bp, b.shape[0],
+        _check(lib().lzhip_get_output_average(self._h, c, bp, b.shape[0],
                                               int(to_move), float(temperature), _ptr(policy),
                                               ctypes.byref(win)))
         del keep
@@ -451,7 +454,7 @@ class HIPScheduler:
         c, keep = _c_heads(heads)
         res = SearchResult()
         moves = (ctypes.c_int * max(int(cfg.moves), 1))()
-        _check(lib().lzhip_selfplay(self._h, ctypes.byref(c), ctypes.byref(cfg), ctypes.byref(res),
+        _check(lib().lzhip_selfplay(self._h, c, ctypes.byref(cfg), ctypes.byref(res),
                                     moves, len(moves)))
         del keep
         return res, list(moves)[:res.moves_played]

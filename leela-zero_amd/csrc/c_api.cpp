@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 
@@ -19,6 +20,10 @@ using namespace lzhip;
 struct lzhip_handle {
     std::unique_ptr<HIPScheduler> sched;
     HIPPipe* pipe = nullptr;  // owned by sched
+    // host-side copy of what lzhip_push_heads received, for the entry points
+    // that run the heads on the calling thread with `heads == NULL`
+    std::shared_ptr<const HeadWeights> host_heads;
+    std::mutex heads_mu;
 };
 
 static thread_local std::string g_err;
@@ -165,6 +170,11 @@ int lzhip_push_heads(lzhip_handle* h, const float* bn_pol_mean, const float* bn_
     HeadWeightsHost hw{bn_pol_mean, bn_pol_scale, ip_pol_w,  ip_pol_b,  bn_val_mean,
                        bn_val_scale, ip1_val_w,   ip1_val_b, ip2_val_w, ip2_val_b};
     h->pipe->push_heads(hw);
+    const lzhip_head_weights c{bn_pol_mean, bn_pol_scale, ip_pol_w,  ip_pol_b,  bn_val_mean,
+                               bn_val_scale, ip1_val_w,   ip1_val_b, ip2_val_w, ip2_val_b};
+    auto host = std::make_shared<const HeadWeights>(c);
+    std::lock_guard<std::mutex> lk(h->heads_mu);
+    h->host_heads = std::move(host);
     return LZHIP_OK;
     GUARD_END
 }
@@ -255,6 +265,19 @@ static bool heads_complete(const lzhip_head_weights* w) {
            w->bn_val_scale && w->ip1_val_w && w->ip1_val_b && w->ip2_val_w && w->ip2_val_b;
 }
 
+// The head parameters an entry point works with: the caller's, or, for NULL,
+// the ones lzhip_push_heads stored.
+static std::shared_ptr<const HeadWeights> resolve_heads(lzhip_handle* h,
+                                                        const lzhip_head_weights* heads) {
+    if (heads) {
+        if (!heads_complete(heads)) throw std::invalid_argument("head parameters contain a null pointer");
+        return std::make_shared<const HeadWeights>(*heads);
+    }
+    std::lock_guard<std::mutex> lk(h->heads_mu);
+    if (!h->host_heads) throw std::invalid_argument("heads is NULL and lzhip_push_heads was not called");
+    return h->host_heads;
+}
+
 int lzhip_symmetry_index(int symmetry, int idx) { return symmetry_index(symmetry, idx); }
 
 int lzhip_gather_features(const uint8_t* boards, int n_boards, int to_move, int symmetry,
@@ -272,18 +295,17 @@ int lzhip_gather_features(const uint8_t* boards, int n_boards, int to_move, int 
 int lzhip_get_output(lzhip_handle* h, const lzhip_head_weights* heads, const uint8_t* boards,
                      int n_boards, int to_move, int symmetry, float softmax_temp, float* policy,
                      float* winrate) {
-    if (!h || !heads_complete(heads) || !boards || !policy || !winrate)
-        return fail(LZHIP_EINVAL, "null argument");
+    if (!h || !boards || !policy || !winrate) return fail(LZHIP_EINVAL, "null argument");
     if (!(softmax_temp > 0.0f)) return fail(LZHIP_EINVAL, "softmax_temp must be positive");
     GUARD_BEGIN
+    const auto hw = resolve_heads(h, heads);
     std::vector<float> in(LZHIP_INPUT_SIZE), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
     const int rc = lzhip_gather_features(boards, n_boards, to_move, symmetry, in.data());
     if (rc != LZHIP_OK) return rc;
     const int frc = h->sched->forward_raw(in.data(), pol.data(), val.data());
     if (frc == LZHIP_EHALT) return fail(LZHIP_EHALT, "halted by drain");
-    const HeadWeights hw(*heads);
     float p[go::kPoints + 1];
-    heads_on_host(hw, pol.data(), val.data(), softmax_temp, p, winrate);
+    heads_on_host(*hw, pol.data(), val.data(), softmax_temp, p, winrate);
     for (int i = 0; i < go::kPoints; i++) policy[symmetry_index(symmetry, i)] = p[i];
     policy[go::kPoints] = p[go::kPoints];
     return LZHIP_OK;
@@ -293,10 +315,10 @@ int lzhip_get_output(lzhip_handle* h, const lzhip_head_weights* heads, const uin
 int lzhip_get_output_average(lzhip_handle* h, const lzhip_head_weights* heads,
                              const uint8_t* boards, int n_boards, int to_move,
                              float softmax_temp, float* policy, float* winrate) {
-    if (!h || !heads_complete(heads) || !boards || !policy || !winrate)
-        return fail(LZHIP_EINVAL, "null argument");
+    if (!h || !boards || !policy || !winrate) return fail(LZHIP_EINVAL, "null argument");
     if (!(softmax_temp > 0.0f)) return fail(LZHIP_EINVAL, "softmax_temp must be positive");
     GUARD_BEGIN
+    const auto hw = resolve_heads(h, heads);
     constexpr int S = 8;
     std::vector<float> in((size_t)S * LZHIP_INPUT_SIZE), pol((size_t)S * LZHIP_POL_SIZE),
         val((size_t)S * LZHIP_VAL_SIZE);
@@ -312,12 +334,11 @@ int lzhip_get_output_average(lzhip_handle* h, const lzhip_head_weights* heads,
                                pol.data() + (size_t)s0 * LZHIP_POL_SIZE,
                                val.data() + (size_t)s0 * LZHIP_VAL_SIZE);
     }
-    const HeadWeights hw(*heads);
     for (int i = 0; i <= go::kPoints; i++) policy[i] = 0.0f;
     float win = 0.0f;
     for (int sym = 0; sym < S; sym++) {
         float p[go::kPoints + 1], w;
-        heads_on_host(hw, pol.data() + (size_t)sym * LZHIP_POL_SIZE,
+        heads_on_host(*hw, pol.data() + (size_t)sym * LZHIP_POL_SIZE,
                       val.data() + (size_t)sym * LZHIP_VAL_SIZE, softmax_temp, p, &w);
         for (int i = 0; i < go::kPoints; i++) policy[symmetry_index(sym, i)] += p[i] / (float)S;
         policy[go::kPoints] += p[go::kPoints] / (float)S;
@@ -351,12 +372,13 @@ int lzhip_search_default_config(lzhip_search_config* cfg) {
 int lzhip_selfplay(lzhip_handle* h, const lzhip_head_weights* heads,
                    const lzhip_search_config* cfg, lzhip_search_result* result, int* moves_out,
                    int moves_cap) {
-    if (!h || !heads_complete(heads) || !cfg || !result) return fail(LZHIP_EINVAL, "null argument");
+    if (!h || !cfg || !result) return fail(LZHIP_EINVAL, "null argument");
     if (cfg->threads < 1 || cfg->threads > 4096 || cfg->visits < 1 || cfg->moves < 0 ||
         !(cfg->softmax_temp > 0.0f))
         return fail(LZHIP_EINVAL, "threads in 1..4096, visits >= 1, moves >= 0, softmax_temp > 0");
     GUARD_BEGIN
-    selfplay(*h->sched, *heads, *cfg, *result, moves_out, moves_out ? moves_cap : 0);
+    selfplay(*h->sched, resolve_heads(h, heads), *cfg, *result, moves_out,
+             moves_out ? moves_cap : 0);
     return LZHIP_OK;
     GUARD_END
 }

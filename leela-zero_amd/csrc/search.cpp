@@ -178,9 +178,9 @@ void EvalCache::clear() {
 // network facade
 // ---------------------------------------------------------------------------
 
-NetworkFacade::NetworkFacade(ForwardPipe& pipe, const lzhip_head_weights& heads,
+NetworkFacade::NetworkFacade(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads,
                              size_t cache_size, float softmax_temp)
-    : m_pipe(pipe), m_heads(heads), m_cache(cache_size), m_temp(softmax_temp) {}
+    : m_pipe(pipe), m_heads(std::move(heads)), m_cache(cache_size), m_temp(softmax_temp) {}
 
 Netresult NetworkFacade::get_output_internal(const go::Position& pos, int symmetry) {
     thread_local std::vector<float> in(LZHIP_INPUT_SIZE), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
@@ -188,7 +188,7 @@ Netresult NetworkFacade::get_output_internal(const go::Position& pos, int symmet
     m_evals++;
     m_pipe.forward(in, pol, val);  // may throw NetworkHaltException
     float policy[kPoints + 1], winrate;
-    heads_on_host(m_heads, pol.data(), val.data(), m_temp, policy, &winrate);
+    heads_on_host(*m_heads, pol.data(), val.data(), m_temp, policy, &winrate);
     Netresult r;
     const int16_t* map = sym_table().idx[symmetry];
     for (int i = 0; i < kPoints; i++) r.policy[map[i]] = policy[i];
@@ -583,14 +583,14 @@ void UCTSearch::advance(int move) {
 // self-play driver
 // ---------------------------------------------------------------------------
 
-void selfplay(ForwardPipe& pipe, const lzhip_head_weights& heads, const lzhip_search_config& cfg,
-              lzhip_search_result& out, int* moves, int moves_cap) {
+void selfplay(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads,
+              const lzhip_search_config& cfg, lzhip_search_result& out, int* moves, int moves_cap) {
     std::memset(&out, 0, sizeof(out));
     auto* sched = dynamic_cast<HIPScheduler*>(&pipe);
     lzhip_stats before{};
     if (sched) before = sched->stats();
 
-    NetworkFacade net(pipe, heads, (size_t)std::max(cfg.cache_size, 0), cfg.softmax_temp);
+    NetworkFacade net(pipe, std::move(heads), (size_t)std::max(cfg.cache_size, 0), cfg.softmax_temp);
     net.set_symmetry_probe(cfg.random_moves == 0);  // as the reference: not in randomised self-play
     UCTSearch search(net, cfg);
     go::Position pos;

@@ -89,8 +89,11 @@ private:
 // The slice of `Network` the search needs.
 class NetworkFacade {
 public:
-    NetworkFacade(ForwardPipe& pipe, const lzhip_head_weights& heads, size_t cache_size,
+    NetworkFacade(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads, size_t cache_size,
                   float softmax_temp);
+    NetworkFacade(ForwardPipe& pipe, const lzhip_head_weights& heads, size_t cache_size,
+                  float softmax_temp)
+        : NetworkFacade(pipe, std::make_shared<const HeadWeights>(heads), cache_size, softmax_temp) {}
     // symmetry in 0..7, or -1 for a random one drawn from `rng_state`.
     Netresult get_output(const go::Position& pos, int symmetry, uint64_t& rng_state,
                          bool use_cache = true);
@@ -111,7 +114,7 @@ public:
 
 private:
     ForwardPipe& m_pipe;
-    HeadWeights m_heads;
+    std::shared_ptr<const HeadWeights> m_heads;
     EvalCache m_cache;
     float m_temp;
     bool m_symmetry_probe = true;
@@ -178,8 +181,13 @@ private:
 
 // Plays cfg.moves moves of self-play from the empty board; fills `out` and, if
 // given, the move list.
-void selfplay(ForwardPipe& pipe, const lzhip_head_weights& heads, const lzhip_search_config& cfg,
-              lzhip_search_result& out, int* moves, int moves_cap);
+void selfplay(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads,
+              const lzhip_search_config& cfg, lzhip_search_result& out, int* moves, int moves_cap);
+inline void selfplay(ForwardPipe& pipe, const lzhip_head_weights& heads,
+                     const lzhip_search_config& cfg, lzhip_search_result& out, int* moves,
+                     int moves_cap) {
+    selfplay(pipe, std::make_shared<const HeadWeights>(heads), cfg, out, moves, moves_cap);
+}
 
 }  // namespace lzhip
 #endif

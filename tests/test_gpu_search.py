@@ -82,6 +82,12 @@ def test_average_ensemble_matches_oracle(pkg, netgen, orc, max_batch):
     assert float(np.abs(policy - want).max()) <= 1e-4
     assert abs(winrate - want_win) <= 1e-4
     assert abs(float(policy.sum()) - 1.0) < 1e-4
+    # heads=None stands for the parameters handed to push_heads
+    with pytest.raises(ValueError):
+        pipe.get_output_average(None, np.array(boards, np.uint8), b.to_move)
+    pipe.push_heads(h)
+    policy2, winrate2 = pipe.get_output_average(None, np.array(boards, np.uint8), b.to_move)
+    assert np.array_equal(policy, policy2) and winrate == winrate2
     # the position is not symmetric, so the mean differs from any single symmetry
     single, _ = pipe.get_output(h, np.array(boards, np.uint8), b.to_move, 0)
     assert float(np.abs(single - policy).max()) > 1e-4
