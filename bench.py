@@ -26,7 +26,7 @@ PEAK_HBM = 8.0e12        # bytes/s
 # size: x2.0 and x1.0); summary and commands in profiles/gemm_and_transform_40x256_fp16_b64_pmc.txt.
 # Counters cannot be read from inside this process, so the figure is only reported for the
 # workload it was measured on: (blocks, filters, precision, batch).
-MEASURED_GEMM_TRAFFIC = {(40, 256, "fp16", 64): (17172.8 * 2.0 + 28800.0 * 1.0) * 1024.0}
+MEASURED_GEMM_TRAFFIC = {(40, 256, "fp16", 64): (17792.3 * 2.0 + 28800.0 * 1.0) * 1024.0}
 
 
 def gemm_flops(batch, filters, n_layers):
@@ -248,7 +248,7 @@ def main():
     peak = PEAK_MFMA_F16 if prec == pkg.FP16 else PEAK_MFMA_F32
     gemm_rate = gf / (ms[pkg.K_GEMM] * 1e-3)
     roofline = {
-        "kernel": "wino_gemm_k (36-way batched Winograd GEMM)",
+        "kernel": "wino_gemm_split_k / wino_gemm_k family (36-way batched Winograd GEMM)",
         "bound": "mfma", "achieved": gemm_rate / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
         "frac": gemm_rate / peak,
         "traffic": MEASURED_GEMM_TRAFFIC.get((blocks, F, args.precision, B)),
