@@ -385,27 +385,35 @@ template <> __device__ __forceinline__ half_t act_to_storage<half_t>(float v) {
 // bounds handling.  Loads that fall outside the board (clipped tiles) read
 // neighbouring memory or, past the end of the buffer, zero (raw buffer
 // semantics); their results are never stored.
-constexpr int kFuseCG = 64;      // channels per workgroup
-constexpr int kFuseWaves = 13;   // 13 x 2 half-waves >= 25 tiles
+//
+// CG = channels per workgroup.  64 (a half-wave per tile, 13 wavefronts) moves
+// whole 128-byte runs and is the choice when there are enough boards to give
+// every compute unit a workgroup; with few boards the kernel is bound by the
+// arithmetic of the one compute unit a workgroup runs on, and 32 or 16 channels
+// per workgroup (4 or 8 tiles per wavefront, 7 or 4 wavefronts) spread a board
+// over more compute units.
 constexpr int kPlane = 22;       // LDS plane: 19 points + 1 zero halo before + 2 after
+constexpr int fuse_waves(int cg) { return (kTilesPerBoard + 128 / cg - 1) / (128 / cg); }
 
-template <typename P>
-__global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
+template <typename P, int CG>
+__global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ act_out,
     P* __restrict__ Vn, const float* __restrict__ bn_scale, const float* __restrict__ bn_mean,
     float rfac, int n, int Kp, int Tp) {
     typedef typename BufIO2<P>::pair_t pair_t;
-    __shared__ pair_t ybuf[kPlane * kPlane * (kFuseCG / 2)];
-    constexpr int CP = kFuseCG / 2;   // channel pairs per plane cell
-    const int ncg = Kp / kFuseCG;
+    constexpr int CP = CG / 2;        // channel pairs per plane cell = lanes per tile
+    constexpr int TPW = 64 / CP;      // tiles per wavefront
+    constexpr int WAVES = fuse_waves(CG);
+    __shared__ pair_t ybuf[kPlane * kPlane * CP];
+    const int ncg = Kp / CG;
     const int b = blockIdx.x / ncg;
     const int cg = blockIdx.x - b * ncg;
 
     const unsigned lane = threadIdx.x & 63;
-    const unsigned cl = lane & 31, sub = lane >> 5;    // channel pair, tile of the pair
+    const unsigned cl = lane % CP, sub = lane / CP;    // channel pair, tile within the wavefront
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const unsigned esz = (unsigned)sizeof(P);
-    const int j = 2 * wave + (int)sub;                 // this lane's tile
+    const int j = TPW * wave + (int)sub;               // this lane's tile
     const bool valid = j < kTilesPerBoard;
     const int jc = valid ? j : kTilesPerBoard - 1;
     const int by = jc / 5, bx = jc - by * 5;
@@ -418,19 +426,19 @@ __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
     const __amdgpu_buffer_rsrc_t rV = make_rsrc(Vn, tile_bytes);
     const __amdgpu_buffer_rsrc_t rR = make_rsrc(res != nullptr ? res : M, act_bytes);
     const __amdgpu_buffer_rsrc_t rA = make_rsrc(act_out != nullptr ? act_out : Vn, act_bytes);
-    // per-lane byte offsets: channel pair (+ one tile row for the upper half-wave) / tile origin
+    // per-lane byte offsets: channel pair (+ the tile's row within the wavefront) / tile origin
     const unsigned voff_t = cl * 2 * esz + (valid ? sub : 0u) * (unsigned)Kp * esz;
     const unsigned voff_a =
         cl * 2 * esz + (unsigned)((4 * by) * kBoard + 4 * bx) * (unsigned)Kp * esz;
     // uniform byte offsets of the wavefront's first tile / of the board
     const unsigned soff_t =
-        ((unsigned)(b * kTilesPerBoard + 2 * wave) * (unsigned)Kp + cg * kFuseCG) * esz;
-    const unsigned soff_a = ((unsigned)(b * kPts) * (unsigned)Kp + cg * kFuseCG) * esz;
+        ((unsigned)(b * kTilesPerBoard + TPW * wave) * (unsigned)Kp + cg * CG) * esz;
+    const unsigned soff_a = ((unsigned)(b * kPts) * (unsigned)Kp + cg * CG) * esz;
     float sc[2], mn[2];
 #pragma unroll
     for (int v = 0; v < 2; v++) {
-        sc[v] = bn_scale[cg * kFuseCG + cl * 2 + v];
-        mn[v] = bn_mean[cg * kFuseCG + cl * 2 + v];
+        sc[v] = bn_scale[cg * CG + cl * 2 + v];
+        mn[v] = bn_mean[cg * CG + cl * 2 + v];
     }
 
     // all loads of the pass go out first
@@ -460,12 +468,12 @@ __global__ __launch_bounds__(kFuseWaves * 64) void out_in_transform_k(
     }
 
     // zero the halo cells of the plane (rows and columns 0, 20, 21): 3 full rows
-    // and 3 cells in each of the 19 rows between them; one cell per half-wave
+    // and 3 cells in each of the 19 rows between them; one cell per tile slot
     {
         pair_t zero;
         zero.x = (P)0.0f;
         zero.y = (P)0.0f;
-        for (int q = 2 * wave + (int)sub; q < 3 * kPlane + 3 * kBoard; q += 2 * kFuseWaves) {
+        for (int q = TPW * wave + (int)sub; q < 3 * kPlane + 3 * kBoard; q += TPW * WAVES) {
             int cell;
             if (q < 3 * kPlane) {
                 const int row = q < kPlane ? 0 : (q < 2 * kPlane ? kBoard + 1 : kBoard + 2);
@@ -559,8 +567,19 @@ template <typename P>
 void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
                              const float* bn_mean, float rfac, int n, int Kp, int Tp,
                              hipStream_t s, LaunchTimer* t) {
-    launch(out_in_transform_k<P>, dim3(n * (Kp / kFuseCG)), dim3(kFuseWaves * 64), s, t, M, res,
-           act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
+    // Enough (board, 64-channel) items to occupy most compute units: wide runs; otherwise
+    // spread (measured at 256 filters: 64 channels wins from batch 48, 32 from batch 8 to
+    // 32, 16 at batch 1).
+    const int items64 = n * (Kp / 64);
+    if (items64 >= 160)
+        launch(out_in_transform_k<P, 64>, dim3(items64), dim3(fuse_waves(64) * 64), s, t, M, res,
+               act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
+    else if (items64 >= 24)
+        launch(out_in_transform_k<P, 32>, dim3(items64 * 2), dim3(fuse_waves(32) * 64), s, t, M,
+               res, act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
+    else
+        launch(out_in_transform_k<P, 16>, dim3(items64 * 4), dim3(fuse_waves(16) * 64), s, t, M,
+               res, act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
 }
 
 // ---------------------------------------------------------------------------
