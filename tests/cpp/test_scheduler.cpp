@@ -137,8 +137,8 @@ static void test_population_batches(int concurrency) {
     CHECK(mean >= 9.0);
 }
 
-static void test_drain_resume() {
-    auto* fe = new FakeExec(4, 20000);  // slow executor: requests pile up in the queue
+static void test_drain_resume(int concurrency) {
+    auto* fe = new FakeExec(4, 20000, concurrency);  // slow executor: requests pile up in the queue
     HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
     s.set_max_wait_us(0);
     std::atomic<int> ok{0}, halted{0};
@@ -160,11 +160,11 @@ static void test_drain_resume() {
     std::printf("drain/resume: %d served, %d halted\n", ok.load(), halted.load());
 }
 
-static void test_destroy_with_waiters() {
+static void test_destroy_with_waiters(int concurrency) {
     std::atomic<int> ok{0}, halted{0};
     std::vector<std::thread> th;
     {
-        auto* fe = new FakeExec(2, 30000);
+        auto* fe = new FakeExec(2, 30000, concurrency);
         auto s = std::make_unique<HIPScheduler>(std::unique_ptr<BatchExecutor>(fe));
         s->set_max_wait_us(0);
         for (int t = 0; t < 8; t++) th.emplace_back([&, t, p = s.get()] { one_call(*p, (float)t, 0.0f, ok, halted); });
@@ -173,12 +173,12 @@ static void test_destroy_with_waiters() {
         for (auto& t : th) t.join();
     }
     CHECK(ok + halted == 8);
-    { HIPScheduler idle{std::unique_ptr<BatchExecutor>(new FakeExec(2, 10))}; }
+    { HIPScheduler idle{std::unique_ptr<BatchExecutor>(new FakeExec(2, 10, concurrency))}; }
     std::printf("destroy: %d served, %d halted\n", ok.load(), halted.load());
 }
 
-static void test_executor_failure() {
-    auto* fe = new FakeExec(4, 10);
+static void test_executor_failure(int concurrency) {
+    auto* fe = new FakeExec(4, 10, concurrency);
     HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
     fe->fail_next = true;
     std::vector<float> in(LZHIP_INPUT_SIZE, 0.0f), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
@@ -211,9 +211,11 @@ int main() {
     test_concurrent(5, 8, 20, 2);
     test_population_batches(1);
     test_population_batches(2);
-    test_drain_resume();
-    test_destroy_with_waiters();
-    test_executor_failure();
+    for (int c = 1; c <= 2; c++) {
+        test_drain_resume(c);
+        test_destroy_with_waiters(c);
+        test_executor_failure(c);
+    }
     std::printf("scheduler tests passed\n");
     return 0;
 }
