@@ -292,7 +292,33 @@ UCTSearch::UCTSearch(NetworkFacade& net, const lzhip_search_config& cfg)
         throw std::invalid_argument("search config: threads, visits >= 1, virtual_loss >= 0");
 }
 
-UCTSearch::~UCTSearch() { free_tree(m_root); }
+UCTSearch::~UCTSearch() {
+    {
+        std::lock_guard<std::mutex> lk(m_pool_mu);
+        m_quit = true;
+    }
+    m_pool_cv.notify_all();
+    for (auto& th : m_pool) th.join();
+    free_tree(m_root);
+}
+
+// Search threads live as long as the search object: every move wakes them with
+// a new generation number instead of creating them again.
+void UCTSearch::pool_thread() {
+    uint64_t seen = 0;
+    std::unique_lock<std::mutex> lk(m_pool_mu);
+    for (;;) {
+        m_pool_cv.wait(lk, [&] { return m_quit || m_generation != seen; });
+        if (m_quit) return;
+        seen = m_generation;
+        const go::Position* root = m_root_pos;
+        const uint64_t seed = next_rand(m_seed);
+        lk.unlock();
+        worker(root, seed);
+        lk.lock();
+        if (--m_active == 0) m_done_cv.notify_all();
+    }
+}
 
 int UCTSearch::root_visits() const { return m_root ? m_root->visits.load() : 0; }
 
@@ -510,10 +536,15 @@ int UCTSearch::think(const go::Position& root) {
 
     if (m_root->visits.load() < m_cfg.visits) {
         m_run = true;
-        std::vector<std::thread> pool;
-        pool.reserve((size_t)m_cfg.threads);
-        for (int t = 0; t < m_cfg.threads; t++)
-            pool.emplace_back(&UCTSearch::worker, this, &root, next_rand(m_seed));
+        {
+            std::lock_guard<std::mutex> lk(m_pool_mu);
+            m_root_pos = &root;
+            m_active = m_cfg.threads;
+            m_generation++;
+            while ((int)m_pool.size() < m_cfg.threads)
+                m_pool.emplace_back(&UCTSearch::pool_thread, this);
+        }
+        m_pool_cv.notify_all();
         // A position in which no simulation can end with a value (every child
         // ruled out by superko) must not spin forever.
         const uint64_t wasted_limit = m_wasted.load() + 1000ull * (uint64_t)m_cfg.visits;
@@ -525,7 +556,10 @@ int UCTSearch::think(const go::Position& root) {
         // are out.
         m_run = false;
         m_net.drain();
-        for (auto& th : pool) th.join();
+        {
+            std::unique_lock<std::mutex> lk(m_pool_mu);
+            m_done_cv.wait(lk, [&] { return m_active == 0; });
+        }
         m_net.resume();
         if (m_failed.load()) throw std::runtime_error(m_failure);
     }

@@ -22,11 +22,13 @@
 
 #include <array>
 #include <atomic>
+#include <condition_variable>
 #include <cstdint>
 #include <deque>
 #include <memory>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -167,6 +169,7 @@ private:
     bool create_children(Node* node, const go::Position& pos, float& eval, uint64_t& rng);
     Child* select_child(Node* node, int color, bool is_root);
     void worker(const go::Position* root, uint64_t seed);
+    void pool_thread();
 
     NetworkFacade& m_net;
     lzhip_search_config m_cfg;
@@ -177,6 +180,14 @@ private:
     std::atomic<uint64_t> m_playouts{0}, m_wasted{0}, m_halted{0}, m_nodes{0};
     SearchStats m_stats;
     uint64_t m_seed;
+    // persistent search threads, woken once per move
+    std::vector<std::thread> m_pool;
+    std::mutex m_pool_mu;
+    std::condition_variable m_pool_cv, m_done_cv;
+    uint64_t m_generation = 0;
+    int m_active = 0;
+    bool m_quit = false;
+    const go::Position* m_root_pos = nullptr;
 };
 
 // Plays cfg.moves moves of self-play from the empty board; fills `out` and, if
