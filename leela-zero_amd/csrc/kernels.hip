@@ -342,6 +342,16 @@ template <> struct BufIO2<float> {
         typedef unsigned u2 __attribute__((ext_vector_type(2)));
         __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u2, v), r, voff, soff, 0);
     }
+    // the pair as stored, no conversion (so that nothing has to wait for the data yet)
+    static __device__ __forceinline__ pair_t load_raw(__amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                      unsigned soff) {
+        float a, b;
+        load(r, voff, soff, a, b);
+        pair_t v;
+        v.x = a;
+        v.y = b;
+        return v;
+    }
 };
 template <> struct BufIO2<half_t> {
     typedef half2v pair_t;
@@ -355,6 +365,10 @@ template <> struct BufIO2<half_t> {
     static __device__ __forceinline__ void store(pair_t v, __amdgpu_buffer_rsrc_t r, unsigned voff,
                                                  unsigned soff) {
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
+    }
+    static __device__ __forceinline__ pair_t load_raw(__amdgpu_buffer_rsrc_t r, unsigned voff,
+                                                      unsigned soff) {
+        return __builtin_bit_cast(pair_t, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
     }
 };
 
@@ -427,9 +441,11 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     const __amdgpu_buffer_rsrc_t rR = make_rsrc(res != nullptr ? res : M, act_bytes);
     const __amdgpu_buffer_rsrc_t rA = make_rsrc(act_out != nullptr ? act_out : Vn, act_bytes);
     // per-lane byte offsets: channel pair (+ the tile's row within the wavefront) / tile origin
-    const unsigned voff_t = cl * 2 * esz + (valid ? sub : 0u) * (unsigned)Kp * esz;
-    const unsigned voff_a =
-        cl * 2 * esz + (unsigned)((4 * by) * kBoard + 4 * bx) * (unsigned)Kp * esz;
+    unsigned voff_t = cl * 2 * esz + (valid ? sub : 0u) * (unsigned)Kp * esz;
+    unsigned voff_a = cl * 2 * esz + (unsigned)((4 * by) * kBoard + 4 * bx) * (unsigned)Kp * esz;
+    // Pin both offsets into registers here: computed later, between the two groups of
+    // loads, their arithmetic waits for the first group's data (a register-reuse hazard).
+    asm volatile("" : "+v"(voff_t), "+v"(voff_a));
     // uniform byte offsets of the wavefront's first tile / of the board
     const unsigned soff_t =
         ((unsigned)(b * kTilesPerBoard + TPW * wave) * (unsigned)Kp + cg * CG) * esz;
@@ -441,7 +457,24 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
         mn[v] = bn_mean[cg * CG + cl * 2 + v];
     }
 
-    // all loads of the pass go out first
+    // All loads of the pass go out first, the skip connection's before M's: it is
+    // needed last, and left after M's the compiler places it behind the first
+    // arithmetic on M, a full memory latency late.
+    pair_t r[16];   // kept as stored: converting here would wait for the data
+    if (res != nullptr) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+                r[i * 4 + jj] = BufIO2<P>::load_raw(
+                    rR, voff_a, soff_a + (unsigned)(i * kBoard + jj) * (unsigned)Kp * esz);
+    } else {
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            r[q].x = (P)0.0f;
+            r[q].y = (P)0.0f;
+        }
+    }
     float m[2][36];
     {
         unsigned so = soff_t;
@@ -450,21 +483,6 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
             BufIO2<P>::load(rM, voff_t, so, m[0][p], m[1][p]);
             so += pstride;
         }
-    }
-    float r[2][16];
-    if (res != nullptr) {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int jj = 0; jj < 4; jj++)
-                BufIO2<P>::load(rR, voff_a,
-                                soff_a + (unsigned)(i * kBoard + jj) * (unsigned)Kp * esz,
-                                r[0][i * 4 + jj], r[1][i * 4 + jj]);
-    } else {
-#pragma unroll
-        for (int v = 0; v < 2; v++)
-#pragma unroll
-            for (int q = 0; q < 16; q++) r[v][q] = 0.0f;
     }
 
     // zero the halo cells of the plane (rows and columns 0, 20, 21): 3 full rows
@@ -489,6 +507,7 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     // ---- phase 1: A^T m A, BN (+ residual), ReLU -> LDS plane (+ memory)
     // plane cell of the tile's patch origin (board row 4by-1, column 4bx-1)
     pair_t* const origin = ybuf + ((4 * by) * kPlane + 4 * bx) * CP + cl;
+    pair_t keep[16];   // this tile's activations, written to memory after the barrier
     {
         float o[2][16];
 #pragma unroll
@@ -510,19 +529,26 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
             for (int jj = 0; jj < 4; jj++) {
                 pair_t sv;
                 sv.x = act_to_storage<P>(
-                    fmaxf(0.0f, sc[0] * (o[0][i * 4 + jj] - mn[0]) + rfac * r[0][i * 4 + jj]));
+                    fmaxf(0.0f, sc[0] * (o[0][i * 4 + jj] - mn[0]) + rfac * (float)r[i * 4 + jj].x));
                 sv.y = act_to_storage<P>(
-                    fmaxf(0.0f, sc[1] * (o[1][i * 4 + jj] - mn[1]) + rfac * r[1][i * 4 + jj]));
-                if (valid && i < ny && jj < nx) {
-                    origin[((i + 1) * kPlane + (jj + 1)) * CP] = sv;
-                    if (act_out != nullptr)
-                        BufIO2<P>::store(sv, rA, voff_a,
-                                         soff_a + (unsigned)(i * kBoard + jj) * (unsigned)Kp * esz);
-                }
+                    fmaxf(0.0f, sc[1] * (o[1][i * 4 + jj] - mn[1]) + rfac * (float)r[i * 4 + jj].y));
+                keep[i * 4 + jj] = sv;
+                if (valid && i < ny && jj < nx) origin[((i + 1) * kPlane + (jj + 1)) * CP] = sv;
             }
         }
     }
     __syncthreads();
+    // The activation leaves only now: stores issued before the barrier would have to be
+    // acknowledged before any wavefront may pass it; here they drain under phase 2.
+    if (act_out != nullptr) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+                if (valid && i < ny && jj < nx)
+                    BufIO2<P>::store(keep[i * 4 + jj], rA, voff_a,
+                                     soff_a + (unsigned)(i * kBoard + jj) * (unsigned)Kp * esz);
+    }
 
     // ---- phase 2: B^T d B of the next layer from the plane in LDS
     {
