@@ -457,10 +457,25 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
         mn[v] = bn_mean[cg * CG + cl * 2 + v];
     }
 
-    // All loads of the pass go out first, the skip connection's before M's: it is
-    // needed last, and left after M's the compiler places it behind the first
-    // arithmetic on M, a full memory latency late.
-    pair_t r[16];   // kept as stored: converting here would wait for the data
+    // All loads of the pass go out before any arithmetic.  M's go first, column by
+    // column of the 6x6 position grid: loads return in issue order at the rate the
+    // memory system delivers them, and the first transform pass works on columns, so it
+    // can start on the first six while the rest are still arriving.  The skip
+    // connection (needed last) follows, left as stored: converting it here would wait
+    // for it.  The scheduling barrier keeps the compiler from sinking those loads behind
+    // the first arithmetic on M.
+    pair_t m[36];   // as stored; converted where used
+#pragma unroll
+    for (int xx = 0; xx < 6; xx++) {
+        unsigned so = soff_t + (unsigned)xx * pstride;
+#pragma unroll
+        for (int row = 0; row < 6; row++) {
+            m[row * 6 + xx] = BufIO2<P>::load_raw(rM, voff_t, so);
+            so += 6u * pstride;
+        }
+        __builtin_amdgcn_sched_barrier(0);   // keep the columns in this order
+    }
+    pair_t r[16];
     if (res != nullptr) {
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -475,15 +490,7 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
             r[q].y = (P)0.0f;
         }
     }
-    float m[2][36];
-    {
-        unsigned so = soff_t;
-#pragma unroll
-        for (int p = 0; p < 36; p++) {
-            BufIO2<P>::load(rM, voff_t, so, m[0][p], m[1][p]);
-            so += pstride;
-        }
-    }
+    __builtin_amdgcn_sched_barrier(0);
 
     // zero the halo cells of the plane (rows and columns 0, 20, 21): 3 full rows
     // and 3 cells in each of the 19 rows between them; one cell per tile slot
@@ -510,19 +517,28 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     pair_t keep[16];   // this tile's activations, written to memory after the barrier
     {
         float o[2][16];
+        float t1[2][24];
+        // column pass in the order the columns arrive (the barrier pins that order)
 #pragma unroll
-        for (int v = 0; v < 2; v++) {
-            float t1[24];
+        for (int xx = 0; xx < 6; xx++) {
 #pragma unroll
-            for (int xx = 0; xx < 6; xx++)
-                at6(m[v][0 + xx], m[v][6 + xx], m[v][12 + xx], m[v][18 + xx], m[v][24 + xx],
-                    m[v][30 + xx], t1[0 + xx], t1[6 + xx], t1[12 + xx], t1[18 + xx]);
+            for (int v = 0; v < 2; v++) {
+                float c[6];
+#pragma unroll
+                for (int row = 0; row < 6; row++)
+                    c[row] = (float)(v == 0 ? m[row * 6 + xx].x : m[row * 6 + xx].y);
+                at6(c[0], c[1], c[2], c[3], c[4], c[5], t1[v][0 + xx], t1[v][6 + xx],
+                    t1[v][12 + xx], t1[v][18 + xx]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int v = 0; v < 2; v++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                at6(t1[i * 6 + 0], t1[i * 6 + 1], t1[i * 6 + 2], t1[i * 6 + 3], t1[i * 6 + 4],
-                    t1[i * 6 + 5], o[v][i * 4 + 0], o[v][i * 4 + 1], o[v][i * 4 + 2],
-                    o[v][i * 4 + 3]);
-        }
+                at6(t1[v][i * 6 + 0], t1[v][i * 6 + 1], t1[v][i * 6 + 2], t1[v][i * 6 + 3],
+                    t1[v][i * 6 + 4], t1[v][i * 6 + 5], o[v][i * 4 + 0], o[v][i * 4 + 1],
+                    o[v][i * 4 + 2], o[v][i * 4 + 3]);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
 #pragma unroll
