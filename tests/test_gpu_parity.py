@@ -310,3 +310,53 @@ def test_graph_replays_match_stream_launches(pkg, netgen, orc):
         assert policy.shape == (5, 362)
     pipe.close()
     plain.close()
+
+
+def test_error_behaviour_on_device(pkg, netgen):
+    """Calls out of order and arguments out of range are refused with an error code and a
+    message, never executed: forward before push_weights, push_weights twice, an even layer
+    count, wrong tensor sizes, empty and oversized batches, bad precision/batch/filter
+    arguments at creation, device heads before push_heads.  The pipe keeps working
+    afterwards."""
+    print("case: error behaviour", flush=True)
+    net = netgen.make_network(1, 64, 5)
+    w, h = netgen.prepare(net)
+    x = netgen.synthetic_inputs(3, seed=2)
+    pipe = pkg.HIPScheduler(pkg.FP32, 2)
+    pipe.initialize(64)
+    with pytest.raises(ValueError):
+        pipe.forward_batch(x[:1])                      # no weights yet
+    with pytest.raises(ValueError):
+        pipe.push_weights(6, 18, 32, w)                # filter count differs from initialize
+    bad = pkg.ForwardPipeWeights()
+    bad.__dict__.update(w.__dict__)
+    bad.m_conv_weights = w.m_conv_weights[:2]          # two layers: not 1 + 2*blocks
+    bad.m_batchnorm_means = w.m_batchnorm_means[:2]
+    bad.m_batchnorm_stddevs = w.m_batchnorm_stddevs[:2]
+    with pytest.raises(ValueError):
+        pipe.push_weights(6, 18, 64, bad)
+    pipe.push_weights(6, 18, 64, w)
+    with pytest.raises(ValueError):
+        pipe.push_weights(6, 18, 64, w)                # twice
+    with pytest.raises(ValueError):
+        pipe.forward_batch(x)                          # 3 > max_batch 2
+    with pytest.raises(ValueError):
+        pipe.forward_batch(np.zeros((0, 18, 361), np.float32))
+    with pytest.raises(ValueError):
+        pipe.forward(np.zeros(100, np.float32))
+    with pytest.raises(ValueError):
+        pipe.evaluate_batch(x[:1])                     # device heads not pushed
+    pol, val = pipe.forward_batch(x[:2])
+    assert np.isfinite(pol).all() and np.isfinite(val).all()
+    assert b"" == pkg.lib().lzhip_last_error()[:0]
+    pipe.close()
+    for args in ((pkg.FP32, 0), (pkg.FP32, 5000), (7, 4)):
+        p = pkg.HIPScheduler(*args)
+        with pytest.raises((ValueError, pkg.LzhipError)):
+            p.initialize(64)
+    p = pkg.HIPScheduler(pkg.FP32, 2)
+    with pytest.raises((ValueError, pkg.LzhipError)):
+        p.initialize(0)
+    p = pkg.HIPScheduler(pkg.FP32, 2, device=99)
+    with pytest.raises(pkg.LzhipError):
+        p.initialize(64)
