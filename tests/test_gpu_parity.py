@@ -360,3 +360,16 @@ def test_error_behaviour_on_device(pkg, netgen):
     p = pkg.HIPScheduler(pkg.FP32, 2, device=99)
     with pytest.raises(pkg.LzhipError):
         p.initialize(64)
+
+
+@pytest.mark.parametrize("precision", [0, 1])
+@pytest.mark.parametrize("filters,batch", [(384, 6), (512, 44), (320, 3)])
+def test_other_widths(pkg, netgen, orc, precision, filters, batch):
+    """Widths other than the benchmark's: 6, 8 and 5 k-slices in fp16 (12, 16, 10 in fp32),
+    with the large-tile GEMM at 512 filters."""
+    print("case: width %d b%d precision=%d" % (filters, batch, precision), flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, filters, 4000 + filters, precision,
+                                       batch)
+    x = netgen.synthetic_inputs(batch, seed=filters)
+    check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=[0, batch - 1])
+    pipe.close()
