@@ -88,6 +88,10 @@ public:
                                      ", this library contains gfx950 code only");
         HIP_CHECK(hipStreamCreate(&m_stream));
         m_Fp = round_up(filters, 64);
+        if (!gemm_supports_channels<P>(m_Fp))
+            throw std::invalid_argument(
+                "unsupported filter count: after rounding up to a multiple of 64, fp16 takes up "
+                "to 512 and 640, 768, 896, 1024; fp32 takes up to 512");
         m_C0p = 64;
         m_Tp = round_up(max_batch * kTilesPerBoard, kTileRowPad);
         const size_t B = (size_t)max_batch;

@@ -39,6 +39,9 @@ template <typename P>
 void launch_in_transform(const P* act, P* V, int n, int Cp, int Tp, hipStream_t s,
                          LaunchTimer* t);
 
+// Whether a GEMM pipeline exists for Cp channels (padded count, multiple of 64).
+template <typename P> bool gemm_supports_channels(int Cp);
+
 // M[p][t][k] = sum_c V[p][t][c] * U[p][k][c]
 // T = real tile rows (25 per board); Tp = allocated rows, a multiple of kTileRowPad.
 template <typename P>

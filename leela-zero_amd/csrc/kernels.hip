@@ -6,6 +6,7 @@
 #include "kernels.h"
 
 #include <cstdlib>
+#include <stdexcept>
 
 #include <hip/hip_ext.h>
 
@@ -1160,7 +1161,8 @@ static void launch_gemm_bn(const P* V, const P* U, P* M, int tiles_m, int Tp, in
 #undef LZ_NK
         default: break;
     }
-    // unreachable for supported widths; the pipe checks the width at creation
+    // the pipe refuses such widths at creation (gemm_supports_channels)
+    throw std::invalid_argument("no GEMM instantiated for this channel count");
 }
 
 // The 256 x 256 tile computed as two 128-row passes.  The stores of the first
@@ -1347,6 +1349,17 @@ static void launch_gemm_big(const P* V, const P* U, P* M, int T, int tiles_m, in
         launch(wino_gemm_big_k<P, NK>, dim3(8 * seg), dim3(512), s, t, V, U, M, T, Tp, Cp, Kp,
                tiles_m, tiles_n, seg);
 }
+
+// Channel counts (multiples of 64) for which a k-slice pipeline is instantiated:
+// 1..8, 10, 12, 14 and 16 slices of 128 bytes.
+template <typename P> bool gemm_supports_channels(int Cp) {
+    constexpr int BK = 128 / (int)sizeof(P);
+    if (Cp < 64 || Cp % 64 != 0) return false;
+    const int nk = Cp / BK;
+    return (nk >= 1 && nk <= 8) || nk == 10 || nk == 12 || nk == 14 || nk == 16;
+}
+template bool gemm_supports_channels<float>(int);
+template bool gemm_supports_channels<half_t>(int);
 
 // T = number of real tile rows (25 per board); Tp (the row count of V and M)
 // must be a multiple of 256.

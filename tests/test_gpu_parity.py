@@ -357,6 +357,10 @@ def test_error_behaviour_on_device(pkg, netgen):
     p = pkg.HIPScheduler(pkg.FP32, 2)
     with pytest.raises((ValueError, pkg.LzhipError)):
         p.initialize(0)
+    for prec, filters in ((pkg.FP32, 576), (pkg.FP16, 576), (pkg.FP16, 1100)):
+        p = pkg.HIPScheduler(prec, 2)
+        with pytest.raises(ValueError):
+            p.initialize(filters)                      # no GEMM pipeline for this width
     p = pkg.HIPScheduler(pkg.FP32, 2, device=99)
     with pytest.raises(pkg.LzhipError):
         p.initialize(64)
