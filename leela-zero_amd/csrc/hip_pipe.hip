@@ -94,6 +94,10 @@ public:
                 "to 512 and 640, 768, 896, 1024; fp32 takes up to 512");
         m_C0p = 64;
         m_Tp = round_up(max_batch * kTilesPerBoard, kTileRowPad);
+        // The transform kernels address V and M through 32-bit buffer offsets.
+        if ((size_t)kPos * m_Tp * m_Fp * sizeof(P) >= ((size_t)1 << 31))
+            throw std::invalid_argument(
+                "max_batch x filters too large: the Winograd tile buffers would exceed 2 GiB");
         const size_t B = (size_t)max_batch;
         m_din.alloc(B * kInPlanes * kPts);
         m_dpol.alloc(B * 2 * kPts);
