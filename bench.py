@@ -173,7 +173,7 @@ def main():
         sys.exit(2)
 
     import torch
-    pkg = entry.load_package()
+    pkg = entry.ensure_built()
     import leela_zero_amd.netgen as netgen
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)

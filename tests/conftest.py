@@ -16,7 +16,7 @@ def pytest_configure(config):
 
 @pytest.fixture(scope="session")
 def pkg():
-    return entry.load_package()
+    return entry.ensure_built()
 
 
 @pytest.fixture(scope="session")

@@ -12,9 +12,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 
 import oracle.go_oracle as G  # noqa: E402
-from __graft_entry__ import load_package  # noqa: E402
+from __graft_entry__ import ensure_built  # noqa: E402
 
-lz = load_package()
+lz = ensure_built()
 
 B, W, E, PASS = G.BLACK, G.WHITE, G.EMPTY, G.PASS
 
