@@ -1149,7 +1149,8 @@ static void launch_gemm_nk(const P* V, const P* U, P* M, int tiles_m, int Tp, in
 }
 
 // Channel counts are multiples of 64, so the number of 128-byte k-slices is
-// Cp/64 for fp16 and Cp/32 for fp32; counts up to 512 channels are instantiated.
+// Cp/64 for fp16 and Cp/32 for fp32; 1..8, 10, 12, 14 and 16 slices are instantiated
+// (every width up to 512 channels in both types, 640..1024 by 128 in fp16).
 template <typename P, int BN>
 static void launch_gemm_bn(const P* V, const P* U, P* M, int tiles_m, int Tp, int Cp, int Kp,
                            hipStream_t s, LaunchTimer* t) {
