@@ -115,10 +115,14 @@ def search_workload(args, pkg, netgen):
     pipe.initialize(F)
     pipe.push_weights(6, 18, F, w)
     h = calibrate_heads(pipe, netgen, h, B)
+    dev = 1 if args.device_heads else 0
+    if dev:
+        pipe.push_heads(h)
     cfg = pkg.SearchConfig.default(threads=args.threads, visits=args.visits, moves=args.moves,
-                                   seed=2027, reuse_tree=0 if args.no_tree_reuse else 1)
+                                   seed=2027, reuse_tree=0 if args.no_tree_reuse else 1,
+                                   device_heads=dev)
     warm = pkg.SearchConfig.default(threads=args.threads, visits=min(200, args.visits), moves=1,
-                                    seed=1)
+                                    seed=1, device_heads=dev)
     pipe.selfplay(h, warm)
     pipe.reset_stats()
     res, moves = pipe.selfplay(h, cfg)
@@ -133,8 +137,9 @@ def search_workload(args, pkg, netgen):
         "data": "synthetic (seeded random weights, FC head weights rescaled to unsaturated "
                 "outputs, self-play from the empty board)",
         "config": {"workload": "%d search threads, max batch %d, %dx%d %s, %d visits/move, "
-                               "%d moves" % (args.threads, B, blocks, F, args.precision,
-                                             args.visits, res.moves_played)},
+                               "%d moves, heads on the %s"
+                               % (args.threads, B, blocks, F, args.precision, args.visits,
+                                  res.moves_played, "device" if dev else "search threads")},
         "batch_fill": fill, "mean_batch": res.sched.requests / max(1, res.sched.batches),
         "max_batch_seen": res.sched.max_batch_seen, "batches": res.sched.batches,
         "playouts": res.playouts, "nn_evals": res.evals,
@@ -163,6 +168,8 @@ def main():
     ap.add_argument("--visits", type=int, default=1600)
     ap.add_argument("--moves", type=int, default=20)
     ap.add_argument("--no-tree-reuse", action="store_true")
+    ap.add_argument("--device-heads", action="store_true",
+                    help="search workload: heads computed on the device, not on the search threads")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy kernel of MIB mebibytes three times "
                          "(known traffic, for scaling the FETCH_SIZE / WRITE_SIZE counters)")

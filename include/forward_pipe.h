@@ -17,6 +17,7 @@
 #include <exception>
 #include <memory>
 #include <mutex>
+#include <stdexcept>
 #include <string>
 #include <thread>
 #include <vector>
@@ -77,6 +78,14 @@ public:
     virtual int max_concurrency() const { return 1; }
     // in [n][18*361] -> pol [n][722], val [n][361]; throws std::runtime_error.
     virtual void forward_batch(int n, const float* in, float* pol, float* val) = 0;
+    // Whether evaluate_heads_batch can be served (head parameters are on board).
+    virtual bool has_heads() const { return false; }
+    // Tower + heads for n positions: policy [n][362] (softmax at `temperature`),
+    // value [n] (tanh output).  Executors without heads on board refuse.
+    virtual void evaluate_heads_batch(int /*n*/, const float* /*in*/, float /*temperature*/,
+                                      float* /*policy*/, float* /*value*/) {
+        throw std::logic_error("this executor does not compute the heads");
+    }
 };
 
 // Device executor: owns the weights and activation buffers of one network on
@@ -118,6 +127,11 @@ public:
     // Pointer form of forward() used by the C ABI; returns LZHIP_OK/LZHIP_EHALT
     // and throws std::runtime_error on executor failure.
     int forward_raw(const float* in, float* pol, float* val);
+    // One position through the queue with the heads computed by the executor
+    // (Network::get_output_internal's arithmetic, reference src/Network.cpp:833-851,
+    // moved behind the pipe): policy [362], *value = tanh output.  Requests of this
+    // kind are batched among themselves.  Same return codes as forward_raw.
+    int evaluate_raw(const float* in, float temperature, float* policy, float* value);
 
     BatchExecutor* executor() { return m_exec.get(); }
     lzhip_stats stats();
@@ -130,14 +144,17 @@ public:
 private:
     struct Request {
         const float* in;
-        float* pol;
-        float* val;
+        float* pol;   // raw policy planes [722], or policy [362] when heads are asked for
+        float* val;   // raw value plane [361], or the value scalar
+        bool heads = false;
+        float temperature = 1.0f;
         std::mutex mu;
         std::condition_variable cv;
         int state = 0;  // 0 pending, 1 done, 2 halted, 3 failed
     };
     void start_worker();
     void worker();
+    int submit(const std::shared_ptr<Request>& req);
 
     int m_precision = LZHIP_FP32, m_max_batch = 1, m_device = 0;
     std::unique_ptr<BatchExecutor> m_exec;

@@ -135,6 +135,15 @@ int lzhip_push_heads(lzhip_handle* h, const float* bn_pol_mean, const float* bn_
 int lzhip_evaluate_batch(lzhip_handle* h, int n, const float* in, float temperature,
                          float* policy, float* value, float* logits, float* pol, float* val);
 
+/* One position through the batching queue with the heads computed on the
+ * device: the whole of Network::get_output_internal's arithmetic (reference
+ * src/Network.cpp:824-851) except the symmetry un-rotation, as one blocking,
+ * thread-safe call.  policy [362] (index 361 = pass), *value = tanh output
+ * (winrate = (1 + value) / 2).  Requests of this kind are batched among
+ * themselves; needs lzhip_push_heads.  Returns LZHIP_EHALT while drained. */
+int lzhip_forward_eval(lzhip_handle* h, const float* in, float temperature, float* policy,
+                       float* value);
+
 /* ---- weight preparation on the host (no device needed) ----------------- */
 
 /* Network::winograd_transform_f (reference src/Network.cpp:159-223):

@@ -46,6 +46,8 @@ typedef struct lzhip_search_config {
     int reuse_tree;    /* keep the chosen subtree between moves                   */
     int random_moves;  /* first N moves sampled in proportion to visits           */
     int virtual_loss;  /* 3                                                        */
+    int device_heads;  /* 1: heads computed on the device (lzhip_forward_eval) instead
+                          of on the search threads; needs lzhip_push_heads          */
     float puct;        /* 0.5                                                      */
     float logpuct;     /* 0.015                                                    */
     float logconst;    /* 1.7                                                      */

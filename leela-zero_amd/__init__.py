@@ -37,7 +37,7 @@ EXPORTS = [
     "lzhip_create", "lzhip_destroy", "lzhip_push_weights", "lzhip_forward",
     "lzhip_forward_batch", "lzhip_forward_batch_device", "lzhip_sync", "lzhip_stream",
     "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats", "lzhip_push_heads",
-    "lzhip_evaluate_batch", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
+    "lzhip_evaluate_batch", "lzhip_forward_eval", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
     "lzhip_debug_layer", "lzhip_get_act_scales", "lzhip_profile_forward", "lzhip_last_error",
     "lzhip_version",
 ]
@@ -84,6 +84,7 @@ class SearchConfig(ctypes.Structure):
     _fields_ = [("threads", ctypes.c_int), ("visits", ctypes.c_int), ("moves", ctypes.c_int),
                 ("cache_size", ctypes.c_int), ("reuse_tree", ctypes.c_int),
                 ("random_moves", ctypes.c_int), ("virtual_loss", ctypes.c_int),
+                ("device_heads", ctypes.c_int),
                 ("puct", ctypes.c_float), ("logpuct", ctypes.c_float),
                 ("logconst", ctypes.c_float), ("fpu_reduction", ctypes.c_float),
                 ("softmax_temp", ctypes.c_float), ("komi", ctypes.c_float),
@@ -142,6 +143,7 @@ def lib():
         L.lzhip_reset_stats.argtypes = [ctypes.c_void_p]
         L.lzhip_push_heads.argtypes = [ctypes.c_void_p] + [_fp] * 10
         L.lzhip_evaluate_batch.argtypes = [ctypes.c_void_p, ctypes.c_int, _fp, ctypes.c_float] + [_fp] * 5
+        L.lzhip_forward_eval.argtypes = [ctypes.c_void_p, _fp, ctypes.c_float, _fp, _fp]
         L.lzhip_winograd_transform_f.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp]
         L.lzhip_process_bn_var.argtypes = [_fp, ctypes.c_int]
         L.lzhip_debug_layer.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int] + [_fp] * 5
@@ -399,6 +401,19 @@ class HIPScheduler:
                 raise ValueError("%s must have %d values" % (name, size))
             arrs.append(a)
         _check(lib().lzhip_push_heads(self._h, *[_ptr(a) for a in arrs]))
+
+    def forward_eval(self, input, temperature=1.0):
+        """One position through the batching queue with the heads computed on the
+        device: returns (policy[362] in NN index order, value = tanh output)."""
+        self._need()
+        x = _f32(input).reshape(-1)
+        if x.size != INPUT_SIZE:
+            raise ValueError("input must have 18*361 values")
+        policy = np.empty(MOVES, dtype=np.float32)
+        value = ctypes.c_float()
+        _check(lib().lzhip_forward_eval(self._h, _ptr(x), float(temperature), _ptr(policy),
+                                        ctypes.byref(value)))
+        return policy, value.value
 
     def evaluate_batch(self, inputs, temperature=1.0, want_raw=False):
         """Tower + heads: returns policy [n][362], value [n] (tanh), logits [n][362]

@@ -188,6 +188,16 @@ int lzhip_evaluate_batch(lzhip_handle* h, int n, const float* in, float temperat
     GUARD_END
 }
 
+int lzhip_forward_eval(lzhip_handle* h, const float* in, float temperature, float* policy,
+                       float* value) {
+    if (!h || !in || !policy || !value) return fail(LZHIP_EINVAL, "null argument");
+    GUARD_BEGIN
+    const int rc = h->sched->evaluate_raw(in, temperature, policy, value);
+    if (rc == LZHIP_EHALT) return fail(LZHIP_EHALT, "halted by drain");
+    return rc;
+    GUARD_END
+}
+
 // Network::winograd_transform_f (reference src/Network.cpp:159-223):
 // U = G f G^T for every (output, channel) filter, written position-major with
 // the output channel fastest: U[(xi*6+nu)][c][o].
@@ -359,6 +369,7 @@ int lzhip_search_default_config(lzhip_search_config* cfg) {
     cfg->reuse_tree = 1;
     cfg->random_moves = 0;
     cfg->virtual_loss = 3;
+    cfg->device_heads = 0;
     cfg->puct = 0.5f;
     cfg->logpuct = 0.015f;
     cfg->logconst = 1.7f;

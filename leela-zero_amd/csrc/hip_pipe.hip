@@ -109,6 +109,8 @@ public:
             sl.din.alloc(B * kInPlanes * kPts);
             sl.dpol.alloc(B * 2 * kPts);
             sl.dval.alloc(B * kPts);
+            sl.dpolicy.alloc(B * 362);
+            sl.dvalue.alloc(B);
             HIP_CHECK(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
         }
         m_act0.alloc(B * kPts * m_C0p);
@@ -137,6 +139,7 @@ public:
 
     int max_batch() const override { return m_max_batch; }
     int max_concurrency() const override { return kIoSlots; }
+    bool has_heads() const override { return m_heads_ready; }
     int filters() const override { return m_filters; }
     int precision() const override { return precision_of<P>(); }
     void* stream() override { return m_stream; }
@@ -209,6 +212,20 @@ public:
     // the lock, so that the next batch is queued on the device while this one
     // runs and host-side copies overlap device work.
     void forward_batch(int n, const float* in, float* pol, float* val) override {
+        run_host_batch(n, in, false, 1.0f, pol, val);
+    }
+
+    // The same path with the heads computed on the device: policy [n][362] and the
+    // tanh value [n] come back instead of the raw planes.
+    void evaluate_heads_batch(int n, const float* in, float temperature, float* policy,
+                              float* value) override {
+        if (!m_heads_ready) throw std::invalid_argument("push_heads has not been called");
+        if (!(temperature > 0.0f)) throw std::invalid_argument("temperature must be positive");
+        run_host_batch(n, in, true, temperature, policy, value);
+    }
+
+    void run_host_batch(int n, const float* in, bool heads, float temperature, float* out_a,
+                        float* out_b) {
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
         IoSlot* sl = nullptr;
@@ -231,25 +248,37 @@ public:
                     std::lock_guard<std::mutex> lk(self->m_slot_mu);
                     sl->busy = false;
                 }
-                self->m_slot_cv.notify_one();
+                self->m_slot_cv.notify_all();
             }
         } release{this, sl};
+        // sizes of the two results per position, staged through hpol / hval
+        const size_t na = heads ? 362 : 2 * kPts, nb = heads ? 1 : kPts;
         std::memcpy(sl->hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
         {
             std::lock_guard<std::mutex> lk(m_mu);
             HIP_CHECK(hipMemcpyAsync(sl->din.p, sl->hin.p, sizeof(float) * (size_t)n * kInPlanes * kPts,
                                      hipMemcpyHostToDevice, m_stream));
             run_forward(n, sl->din.p, sl->dpol.p, sl->dval.p);
+            const float* da = sl->dpol.p;
+            const float* db = sl->dval.p;
+            if (heads) {
+                HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
+                              m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
+                launch_heads(sl->dpol.p, sl->dval.p, hp, temperature, sl->dpolicy.p, nullptr,
+                             sl->dvalue.p, n, m_stream);
+                da = sl->dpolicy.p;
+                db = sl->dvalue.p;
+            }
             HIP_CHECK(hipGetLastError());
-            HIP_CHECK(hipMemcpyAsync(sl->hpol.p, sl->dpol.p, sizeof(float) * (size_t)n * 2 * kPts,
+            HIP_CHECK(hipMemcpyAsync(sl->hpol.p, da, sizeof(float) * (size_t)n * na,
                                      hipMemcpyDeviceToHost, m_stream));
-            HIP_CHECK(hipMemcpyAsync(sl->hval.p, sl->dval.p, sizeof(float) * (size_t)n * kPts,
+            HIP_CHECK(hipMemcpyAsync(sl->hval.p, db, sizeof(float) * (size_t)n * nb,
                                      hipMemcpyDeviceToHost, m_stream));
             HIP_CHECK(hipEventRecord(sl->done, m_stream));
         }
         HIP_CHECK(hipEventSynchronize(sl->done));
-        std::memcpy(pol, sl->hpol.p, sizeof(float) * (size_t)n * 2 * kPts);
-        std::memcpy(val, sl->hval.p, sizeof(float) * (size_t)n * kPts);
+        std::memcpy(out_a, sl->hpol.p, sizeof(float) * (size_t)n * na);
+        std::memcpy(out_b, sl->hval.p, sizeof(float) * (size_t)n * nb);
     }
 
     // -------------------------------------------------------------------
@@ -262,11 +291,19 @@ public:
         };
         up(m_h[0], hw.bn_pol_mean, 2);
         up(m_h[1], hw.bn_pol_scale, 2);
-        up(m_h[2], hw.ip_pol_w, (size_t)362 * 722);
+        {   // FC matrices go up input-major (what heads_k reads)
+            std::vector<float> t((size_t)722 * 362);
+            for (int o = 0; o < 362; o++)
+                for (int i = 0; i < 722; i++) t[(size_t)i * 362 + o] = hw.ip_pol_w[(size_t)o * 722 + i];
+            up(m_h[2], t.data(), t.size());
+            t.assign((size_t)361 * 256, 0.0f);
+            for (int o = 0; o < 256; o++)
+                for (int i = 0; i < 361; i++) t[(size_t)i * 256 + o] = hw.ip1_val_w[(size_t)o * 361 + i];
+            up(m_h[6], t.data(), t.size());
+        }
         up(m_h[3], hw.ip_pol_b, 362);
         up(m_h[4], hw.bn_val_mean, 1);
         up(m_h[5], hw.bn_val_scale, 1);
-        up(m_h[6], hw.ip1_val_w, (size_t)256 * 361);
         up(m_h[7], hw.ip1_val_b, 256);
         up(m_h[8], hw.ip2_val_w, 256);
         up(m_h[9], hw.ip2_val_b, 1);
@@ -593,7 +630,7 @@ private:
     // "copied out" at once; their device work is ordered by the one stream.
     struct IoSlot {
         PinnedBuf<float> hin, hpol, hval;
-        DevBuf<float> din, dpol, dval;
+        DevBuf<float> din, dpol, dval, dpolicy, dvalue;
         hipEvent_t done = nullptr;
         bool busy = false;
     };

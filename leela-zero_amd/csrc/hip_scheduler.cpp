@@ -116,14 +116,31 @@ void HIPScheduler::forward(const std::vector<float>& input, std::vector<float>& 
 }
 
 int HIPScheduler::forward_raw(const float* in, float* pol, float* val) {
-    if (m_draining.load()) {
-        m_halted++;
-        return LZHIP_EHALT;
-    }
     auto req = std::make_shared<Request>();
     req->in = in;
     req->pol = pol;
     req->val = val;
+    return submit(req);
+}
+
+int HIPScheduler::evaluate_raw(const float* in, float temperature, float* policy, float* value) {
+    if (!(temperature > 0.0f)) throw std::invalid_argument("temperature must be positive");
+    if (!m_exec || !m_exec->has_heads())
+        throw std::invalid_argument("the executor holds no head parameters (push_heads)");
+    auto req = std::make_shared<Request>();
+    req->in = in;
+    req->pol = policy;
+    req->val = value;
+    req->heads = true;
+    req->temperature = temperature;
+    return submit(req);
+}
+
+int HIPScheduler::submit(const std::shared_ptr<Request>& req) {
+    if (m_draining.load()) {
+        m_halted++;
+        return LZHIP_EHALT;
+    }
     m_outstanding++;
     {
         std::lock_guard<std::mutex> lk(m_mutex);
@@ -228,7 +245,12 @@ void HIPScheduler::worker() {
                 if (!m_running) return;
             }
             // drain() may have emptied the queue while we waited
+            // a batch holds requests of one kind (raw planes, or heads at one temperature)
             while (!m_queue.empty() && (int)batch.size() < m_max_batch) {
+                const Request& f = *m_queue.front();
+                if (!batch.empty() && (f.heads != batch[0]->heads ||
+                                       (f.heads && f.temperature != batch[0]->temperature)))
+                    break;
                 batch.push_back(std::move(m_queue.front()));
                 m_queue.pop_front();
             }
@@ -241,7 +263,11 @@ void HIPScheduler::worker() {
         int outcome = 1;
         const auto t0 = std::chrono::steady_clock::now();
         try {
-            m_exec->forward_batch(n, in.data(), pol.data(), val.data());
+            if (batch[0]->heads)
+                m_exec->evaluate_heads_batch(n, in.data(), batch[0]->temperature, pol.data(),
+                                             val.data());
+            else
+                m_exec->forward_batch(n, in.data(), pol.data(), val.data());
         } catch (const std::exception& e) {
             outcome = 3;
             std::lock_guard<std::mutex> lk(m_mutex);
@@ -263,7 +289,10 @@ void HIPScheduler::worker() {
         while ((uint32_t)n > seen && !m_max_seen.compare_exchange_weak(seen, (uint32_t)n)) {}
         for (int i = 0; i < n; i++) {
             Request& r = *batch[i];
-            if (outcome == 1) {
+            if (outcome == 1 && r.heads) {
+                std::memcpy(r.pol, pol.data() + (size_t)i * 362, sizeof(float) * 362);
+                *r.val = val[i];
+            } else if (outcome == 1) {
                 std::memcpy(r.pol, pol.data() + (size_t)i * kPolSize, sizeof(float) * kPolSize);
                 std::memcpy(r.val, val.data() + (size_t)i * kValSize, sizeof(float) * kValSize);
             }

@@ -73,9 +73,11 @@ template <typename P>
 void launch_absmax(const P* x, size_t count, float* out, hipStream_t s);
 
 // Head arithmetic above the pipe boundary, one workgroup per position.
+// Device pointers; the two large FC matrices are held input-major:
+// ip_pol_wt [722][362], ip1_val_wt [361][256].
 struct HeadParams {
-    const float *bn_pol_mean, *bn_pol_scale, *ip_pol_w, *ip_pol_b;
-    const float *bn_val_mean, *bn_val_scale, *ip1_val_w, *ip1_val_b, *ip2_val_w, *ip2_val_b;
+    const float *bn_pol_mean, *bn_pol_scale, *ip_pol_wt, *ip_pol_b;
+    const float *bn_val_mean, *bn_val_scale, *ip1_val_wt, *ip1_val_b, *ip2_val_w, *ip2_val_b;
 };
 void launch_heads(const float* pol, const float* val, HeadParams hp, float temperature,
                   float* policy, float* logits, float* value, int n, hipStream_t s);

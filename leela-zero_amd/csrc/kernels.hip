@@ -1472,79 +1472,141 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-__global__ __launch_bounds__(256) void heads_k(const float* __restrict__ pol,
-                                               const float* __restrict__ val, HeadParams hp,
-                                               float temperature, float* __restrict__ policy,
-                                               float* __restrict__ logits,
-                                               float* __restrict__ value) {
-    __shared__ float xin[2 * kPts];
-    __shared__ float lg[362];
-    __shared__ float h1[256];
-    __shared__ float red[8];
-    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// kHeadPB positions per workgroup share every weight they read.  Thread o owns
+// output o of a fully connected layer and walks the inputs in order, reading
+// the input-major copy of the weights (consecutive threads, consecutive
+// addresses) and the activations as LDS broadcasts; the input range is cut in
+// kHeadSplit pieces taken by separate thread groups, whose partial sums meet in
+// LDS, to shorten the chain of dependent multiply-adds.
+constexpr int kHeadPB = 4;
+constexpr int kHeadGroup = 384;     // >= 362 policy outputs, >= 256 hidden units
+constexpr int kHeadSplit = 2;       // thread groups that share an output's input range
+constexpr int kHeadThreads = kHeadGroup * kHeadSplit;
 
-    // ---- policy
-    for (int i = tid; i < 2 * kPts; i += 256) {
-        const int pl = i / kPts;
-        xin[i] = fmaxf(0.0f, hp.bn_pol_scale[pl] * (pol[(size_t)b * 2 * kPts + i] -
-                                                    hp.bn_pol_mean[pl]));
+__global__ __launch_bounds__(kHeadThreads) void heads_k(const float* __restrict__ pol,
+                                                        const float* __restrict__ val,
+                                                        HeadParams hp, float temperature,
+                                                        float* __restrict__ policy,
+                                                        float* __restrict__ logits,
+                                                        float* __restrict__ value, int n) {
+    __shared__ float xin[kHeadPB][2 * kPts];
+    __shared__ float part[kHeadSplit][kHeadPB][364];
+    __shared__ float hv[kHeadPB][256];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = tid / kHeadGroup, o = tid - grp * kHeadGroup;   // input range, output
+    const int b0 = blockIdx.x * kHeadPB;
+    const int nb = min(kHeadPB, n - b0);
+
+    // ---- policy: BN + ReLU, FC 722 -> 362, softmax
+    for (int i = tid; i < kHeadPB * 2 * kPts; i += kHeadThreads) {
+        const int pb = i / (2 * kPts), k = i - pb * (2 * kPts), pl = k / kPts;
+        xin[pb][k] = pb < nb ? fmaxf(0.0f, hp.bn_pol_scale[pl] *
+                                               (pol[(size_t)(b0 + pb) * 2 * kPts + k] -
+                                                hp.bn_pol_mean[pl]))
+                             : 0.0f;
     }
     __syncthreads();
-    for (int o = wave; o < 362; o += 4) {
-        const float* w = hp.ip_pol_w + (size_t)o * (2 * kPts);
+    if (o < 362) {
+        float acc[kHeadPB];
+#pragma unroll
+        for (int pb = 0; pb < kHeadPB; pb++) acc[pb] = grp == 0 ? hp.ip_pol_b[o] : 0.0f;
+        constexpr int span = 2 * kPts / kHeadSplit;
+        const float* w = hp.ip_pol_wt + (size_t)grp * span * 362 + o;
+#pragma unroll 8
+        for (int k = 0; k < span; k++) {
+            const float wk = w[(size_t)k * 362];
+#pragma unroll
+            for (int pb = 0; pb < kHeadPB; pb++) acc[pb] += wk * xin[pb][grp * span + k];
+        }
+#pragma unroll
+        for (int pb = 0; pb < kHeadPB; pb++) part[grp][pb][o] = acc[pb];
+    }
+    __syncthreads();
+    if (wave < nb) {   // one wavefront per position
+        const int pb = wave;
+        float l[6], m = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < 6; q++) {
+            const int i = lane + 64 * q;
+            l[q] = -INFINITY;
+            if (i < 362) {
+                l[q] = part[0][pb][i];
+#pragma unroll
+                for (int g = 1; g < kHeadSplit; g++) l[q] += part[g][pb][i];
+            }
+            m = fmaxf(m, l[q]);
+        }
+        m = wave_max(m);
+        float e[6];
         float s = 0.0f;
-        for (int i = lane; i < 2 * kPts; i += 64) s += w[i] * xin[i];
+#pragma unroll
+        for (int q = 0; q < 6; q++) {
+            e[q] = lane + 64 * q < 362 ? expf((l[q] - m) / temperature) : 0.0f;
+            s += e[q];
+        }
         s = wave_sum(s);
-        if (lane == 0) lg[o] = hp.ip_pol_b[o] + s;
-    }
-    __syncthreads();
-    float m = -INFINITY;
-    for (int i = tid; i < 362; i += 256) m = fmaxf(m, lg[i]);
-    m = wave_max(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
-    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    float e[2];
-    float s = 0.0f;
-    for (int i = tid, q = 0; i < 362; i += 256, q++) {
-        e[q] = expf((lg[i] - m) / temperature);
-        s += e[q];
-    }
-    s = wave_sum(s);
-    if (lane == 0) red[4 + wave] = s;
-    __syncthreads();
-    const float denom = (red[4] + red[5]) + (red[6] + red[7]);
-    for (int i = tid, q = 0; i < 362; i += 256, q++) {
-        policy[(size_t)b * 362 + i] = e[q] / denom;
-        if (logits != nullptr) logits[(size_t)b * 362 + i] = lg[i];
+#pragma unroll
+        for (int q = 0; q < 6; q++) {
+            const int i = lane + 64 * q;
+            if (i < 362) {
+                policy[(size_t)(b0 + pb) * 362 + i] = e[q] / s;
+                if (logits != nullptr) logits[(size_t)(b0 + pb) * 362 + i] = l[q];
+            }
+        }
     }
     __syncthreads();
 
-    // ---- value
-    for (int i = tid; i < kPts; i += 256)
-        xin[i] = fmaxf(0.0f, hp.bn_val_scale[0] * (val[(size_t)b * kPts + i] -
-                                                   hp.bn_val_mean[0]));
-    __syncthreads();
-    for (int o = wave; o < 256; o += 4) {
-        const float* w = hp.ip1_val_w + (size_t)o * kPts;
-        float acc = 0.0f;
-        for (int i = lane; i < kPts; i += 64) acc += w[i] * xin[i];
-        acc = wave_sum(acc);
-        if (lane == 0) h1[o] = fmaxf(0.0f, hp.ip1_val_b[o] + acc);
+    // ---- value: BN + ReLU, FC 361 -> 256 + ReLU, FC 256 -> 1, tanh
+    for (int i = tid; i < kHeadPB * kPts; i += kHeadThreads) {
+        const int pb = i / kPts, k = i - pb * kPts;
+        xin[pb][k] = pb < nb ? fmaxf(0.0f, hp.bn_val_scale[0] *
+                                               (val[(size_t)(b0 + pb) * kPts + k] -
+                                                hp.bn_val_mean[0]))
+                             : 0.0f;
     }
     __syncthreads();
-    if (wave == 0) {
+    if (o < 256) {
+        float acc[kHeadPB];
+#pragma unroll
+        for (int pb = 0; pb < kHeadPB; pb++) acc[pb] = grp == 0 ? hp.ip1_val_b[o] : 0.0f;
+        // 361 inputs: the first group takes 181, the second 180
+        constexpr int span0 = (kPts + kHeadSplit - 1) / kHeadSplit;
+        const int k0 = grp * span0, k1 = min(kPts, k0 + span0);
+        const float* w = hp.ip1_val_wt + o;
+#pragma unroll 8
+        for (int k = k0; k < k1; k++) {
+            const float wk = w[(size_t)k * 256];
+#pragma unroll
+            for (int pb = 0; pb < kHeadPB; pb++) acc[pb] += wk * xin[pb][k];
+        }
+#pragma unroll
+        for (int pb = 0; pb < kHeadPB; pb++) part[grp][pb][o] = acc[pb];
+    }
+    __syncthreads();
+    if (tid < 256) {
+        const float w2 = hp.ip2_val_w[tid];
+#pragma unroll
+        for (int pb = 0; pb < kHeadPB; pb++) {
+            float h = part[0][pb][tid];
+#pragma unroll
+            for (int g = 1; g < kHeadSplit; g++) h += part[g][pb][tid];
+            hv[pb][tid] = fmaxf(0.0f, h) * w2;
+        }
+    }
+    __syncthreads();
+    if (wave < nb) {
+        const int pb = wave;
         float acc = 0.0f;
-        for (int i = lane; i < 256; i += 64) acc += hp.ip2_val_w[i] * h1[i];
+        for (int i = lane; i < 256; i += 64) acc += hv[pb][i];
         acc = wave_sum(acc);
-        if (lane == 0) value[b] = tanhf(hp.ip2_val_b[0] + acc);
+        if (lane == 0) value[b0 + pb] = tanhf(hp.ip2_val_b[0] + acc);
     }
 }
 
 void launch_heads(const float* pol, const float* val, HeadParams hp, float temperature,
                   float* policy, float* logits, float* value, int n, hipStream_t s) {
-    hipLaunchKernelGGL(heads_k, dim3(n), dim3(256), 0, s, pol, val, hp, temperature, policy,
-                       logits, value);
+    hipLaunchKernelGGL(heads_k, dim3((n + kHeadPB - 1) / kHeadPB), dim3(kHeadThreads), 0, s, pol,
+                       val, hp, temperature, policy, logits, value, n);
 }
 
 // ---------------------------------------------------------------------------

@@ -182,13 +182,27 @@ NetworkFacade::NetworkFacade(ForwardPipe& pipe, std::shared_ptr<const HeadWeight
                              size_t cache_size, float softmax_temp)
     : m_pipe(pipe), m_heads(std::move(heads)), m_cache(cache_size), m_temp(softmax_temp) {}
 
+void NetworkFacade::set_device_heads(bool on) {
+    m_sched_heads = nullptr;
+    if (!on) return;
+    m_sched_heads = dynamic_cast<HIPScheduler*>(&m_pipe);
+    if (!m_sched_heads) throw std::invalid_argument("device heads need a HIPScheduler backend");
+}
+
 Netresult NetworkFacade::get_output_internal(const go::Position& pos, int symmetry) {
     thread_local std::vector<float> in(LZHIP_INPUT_SIZE), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
     gather_features(pos, symmetry, in.data());
     m_evals++;
-    m_pipe.forward(in, pol, val);  // may throw NetworkHaltException
     float policy[kPoints + 1], winrate;
-    heads_on_host(*m_heads, pol.data(), val.data(), m_temp, policy, &winrate);
+    if (m_sched_heads) {
+        float value;
+        if (m_sched_heads->evaluate_raw(in.data(), m_temp, policy, &value) == LZHIP_EHALT)
+            throw NetworkHaltException();
+        winrate = (1.0f + value) / 2.0f;
+    } else {
+        m_pipe.forward(in, pol, val);  // may throw NetworkHaltException
+        heads_on_host(*m_heads, pol.data(), val.data(), m_temp, policy, &winrate);
+    }
     Netresult r;
     const int16_t* map = sym_table().idx[symmetry];
     for (int i = 0; i < kPoints; i++) r.policy[map[i]] = policy[i];
@@ -626,6 +640,7 @@ void selfplay(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads,
 
     NetworkFacade net(pipe, std::move(heads), (size_t)std::max(cfg.cache_size, 0), cfg.softmax_temp);
     net.set_symmetry_probe(cfg.random_moves == 0);  // as the reference: not in randomised self-play
+    net.set_device_heads(cfg.device_heads != 0);
     UCTSearch search(net, cfg);
     go::Position pos;
     const auto t0 = std::chrono::steady_clock::now();

@@ -105,6 +105,10 @@ public:
     // its seven symmetric images (their cached policy is mapped back).
     bool probe_cache(const go::Position& pos, Netresult& out);
     void set_symmetry_probe(bool on) { m_symmetry_probe = on; }
+    // Let the backend compute the heads (the pipe must be a HIPScheduler whose
+    // executor has them); the calling thread then only gathers planes and
+    // rotates the policy back.
+    void set_device_heads(bool on);
     void drain() { m_pipe.drain(); }
     void resume() { m_pipe.resume(); }
     EvalCache& cache() { return m_cache; }
@@ -120,6 +124,7 @@ private:
     EvalCache m_cache;
     float m_temp;
     bool m_symmetry_probe = true;
+    HIPScheduler* m_sched_heads = nullptr;   // set when the backend computes the heads
     std::atomic<uint64_t> m_evals{0}, m_probes{0}, m_probe_hits{0};
 };
 

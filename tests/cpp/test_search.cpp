@@ -16,6 +16,9 @@
 //     the seven symmetric images of a cached position, with the policy mapped
 //     back to the asking position's board order;
 //   * a finished game (two passes) is not searched;
+//   * with the heads computed behind the pipe (requests of that kind are batched
+//     among themselves) the search plays the same single-thread game as with the
+//     heads on the calling thread;
 //   * an executor failure reaches the caller as an exception.
 #include <atomic>
 #include <chrono>
@@ -77,8 +80,25 @@ public:
         batches++;
         positions += n;
     }
+    // the heads behind the pipe: same arithmetic as the search threads would do
+    bool has_heads() const override { return host_heads != nullptr; }
+    void evaluate_heads_batch(int n, const float* in, float temperature, float* policy,
+                              float* value) override {
+        if (!host_heads) throw std::logic_error("no heads");
+        std::vector<float> pol((size_t)n * LZHIP_POL_SIZE), val((size_t)n * LZHIP_VAL_SIZE);
+        forward_batch(n, in, pol.data(), val.data());
+        for (int b = 0; b < n; b++) {
+            float win;
+            heads_on_host(*host_heads, pol.data() + (size_t)b * LZHIP_POL_SIZE,
+                          val.data() + (size_t)b * LZHIP_VAL_SIZE, temperature,
+                          policy + (size_t)b * 362, &win);
+            value[b] = 2.0f * win - 1.0f;
+        }
+        head_batches++;
+    }
     std::atomic<bool> fail{false};
-    std::atomic<long> batches{0}, positions{0};
+    std::atomic<long> batches{0}, positions{0}, head_batches{0};
+    std::shared_ptr<const HeadWeights> host_heads;
 
 private:
     int m_mb, m_delay;
@@ -240,6 +260,52 @@ static std::vector<int> play_game(int threads, int visits, int moves, int delay_
     return game;
 }
 
+static void test_heads_behind_the_pipe() {
+    Heads heads;
+    std::vector<int> games[2];
+    for (int mode = 0; mode < 2; mode++) {
+        auto exec = std::make_unique<NeighbourNet>(4, 0);
+        exec->host_heads = std::make_shared<const HeadWeights>(heads.c);
+        NeighbourNet* raw = exec.get();
+        HIPScheduler sched(std::move(exec));
+        lzhip_search_config cfg = config(1, 80, 5);
+        cfg.device_heads = mode;
+        lzhip_search_result res;
+        int moves[5];
+        selfplay(sched, heads.c, cfg, res, moves, 5);
+        games[mode].assign(moves, moves + res.moves_played);
+        CHECK((raw->head_batches.load() > 0) == (mode == 1));
+    }
+    CHECK(games[0] == games[1]);
+    // several threads, both kinds of request in the queue at once
+    auto exec = std::make_unique<NeighbourNet>(8, 100);
+    exec->host_heads = std::make_shared<const HeadWeights>(heads.c);
+    HIPScheduler sched(std::move(exec));
+    std::atomic<int> ok{0};
+    std::vector<std::thread> th;
+    for (int t = 0; t < 8; t++)
+        th.emplace_back([&, t] {
+            std::vector<float> in(LZHIP_INPUT_SIZE, 0.0f), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
+            in[8 * kPoints + 40 + t] = 1.0f;   // one opponent stone
+            for (int r = 0; r < 20; r++) {
+                if ((t + r) & 1) {
+                    float policy[362], value;
+                    CHECK(sched.evaluate_raw(in.data(), 1.0f, policy, &value) == LZHIP_OK);
+                    float sum = 0.0f;
+                    for (float p : policy) sum += p;
+                    CHECK(std::fabs(sum - 1.0f) < 1e-4f);
+                    CHECK(policy[40 + t + 1] > 0.04f && value < 0.0f);
+                } else {
+                    sched.forward(in, pol, val);
+                    CHECK(pol[40 + t + 1] == 3.0f);
+                }
+                ok++;
+            }
+        });
+    for (auto& t : th) t.join();
+    CHECK(ok == 160);
+}
+
 static void test_single_thread_deterministic() {
     lzhip_search_result a{}, b{};
     const auto g1 = play_game(1, 120, 6, 0, 4, &a);
@@ -334,6 +400,8 @@ int main() {
     test_unrotation();
     std::printf("symmetric cache probe\n");
     test_symmetric_cache_probe();
+    std::printf("heads behind the pipe\n");
+    test_heads_behind_the_pipe();
     std::printf("single thread\n");
     test_single_thread_deterministic();
     std::printf("many threads\n");

@@ -128,6 +128,62 @@ def test_selfplay_on_device(pkg, netgen, orc):
     pipe.close()
 
 
+@pytest.mark.parametrize("precision", [0, 1])
+def test_forward_eval_matches_oracle_heads(pkg, netgen, orc, precision):
+    """One position through the queue with the heads on the device, from several threads
+    at once and mixed with raw requests: policy and value against the oracle's heads."""
+    import threading
+    print("case: forward_eval precision=%d" % precision, flush=True)
+    pipe, h, ref, h_ref = make(pkg, netgen, orc, 2, 64, 17, precision, 4)
+    x = netgen.synthetic_inputs(10, seed=4)
+    with pytest.raises(ValueError):
+        pipe.forward_eval(x[0])                       # heads not pushed yet
+    pipe.push_heads(h)
+    orc.use_builtin()
+    tol = 1e-4 if precision == 0 else 2e-2
+    want = []
+    for i in range(10):
+        rp, rv = ref.forward(x[i])
+        want.append(orc.heads(h_ref, rp, rv))
+    errs, raw = [0.0] * 10, [None] * 10
+
+    def work(i):
+        policy, value = pipe.forward_eval(x[i])
+        errs[i] = max(float(np.abs(policy - want[i]["policy"]).max()),
+                      abs(value - want[i]["value"]))
+        raw[i] = pipe.forward(x[i])                   # a raw request in the same queue
+
+    th = [threading.Thread(target=work, args=(i,)) for i in range(10)]
+    [t.start() for t in th]
+    [t.join() for t in th]
+    assert max(errs) <= tol, errs
+    pol, val = pipe.forward_batch(x[:4])
+    for i in range(4):
+        assert np.array_equal(raw[i][0], pol[i]) and np.array_equal(raw[i][1], val[i])
+    with pytest.raises(ValueError):
+        pipe.forward_eval(x[0], temperature=0.0)
+    pipe.close()
+
+
+def test_selfplay_with_device_heads(pkg, netgen, orc):
+    """The search driver with the heads behind the pipe: one thread plays the same game as
+    with the heads on the search thread (fp32: the two head implementations agree far
+    below anything that could flip a visit count on this small net)."""
+    print("case: selfplay device heads", flush=True)
+    pipe, h, ref, h_ref = make(pkg, netgen, orc, 2, 64, 21, 0, 8)
+    pipe.push_heads(h)
+    cfg = pkg.SearchConfig.default(threads=1, visits=60, moves=4, seed=5)
+    r0, m0 = pipe.selfplay(h, cfg)
+    cfg.device_heads = 1
+    r1, m1 = pipe.selfplay(None, cfg)
+    assert m0 == m1 and r0.playouts == r1.playouts
+    cfg = pkg.SearchConfig.default(threads=12, visits=200, moves=4, seed=3, device_heads=1)
+    res, moves = pipe.selfplay(None, cfg)
+    assert res.moves_played == 4 and res.sched.max_batch_seen >= 2
+    assert res.sched.requests + res.sched.halted == res.evals
+    pipe.close()
+
+
 def test_selfplay_argument_checks(pkg, netgen, orc):
     print("case: selfplay argument checks", flush=True)
     pipe, h, ref, h_ref = make(pkg, netgen, orc, 1, 64, 2, 0, 2)
