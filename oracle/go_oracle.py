@@ -12,10 +12,15 @@ board and of `Network`'s input encoding, written for clarity, not speed:
   get_symmetry, :518-531 symmetry_nn_idx_table, :913-966 gather_features).
 
 Pinned by tests/test_search_host.py against hand-worked positions (corner
-capture, ko, snapback, suicide, a sending-two-returning-one repetition, small
-scored boards), against closed forms of the symmetry group, and against each
-other on random games.
+capture, ko, a one-stone capture that is no ko, suicide, a repetition through
+passes, small scored boards), against closed forms of the symmetry group, and,
+where the reference tree is at hand, against the reference's own board code
+compiled from its sources (oracle/Makefile target `ref`, oracle/_ref/ref_board)
+on every ply of random games.
 """
+import os
+import subprocess
+
 N = 19
 NPTS = N * N
 PASS = NPTS
@@ -148,3 +153,54 @@ def gather_features(boards, to_move, symmetry):
             planes[plane][idx] = 1.0
     planes[16 if to_move == BLACK else 17] = [1.0] * NPTS
     return planes
+
+
+# ---- the reference's own board code, when it has been built (oracle/Makefile, target ref)
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REF_BOARD = os.path.join(HERE, "_ref", "ref_board")
+REF_CACHE = os.path.join(HERE, "_ref", "ref_cache")
+REF_SRC = "/root/reference/src"
+
+
+def build_ref_board():
+    """Builds oracle/_ref/ref_board from the reference tree if that tree is present.
+    Returns the path, or None when neither the binary nor the tree exists."""
+    if os.path.exists(os.path.join(REF_SRC, "FullBoard.cpp")):
+        r = subprocess.run(["make", "-C", HERE, "ref"], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("building the reference board failed:\n" + r.stderr)
+    return REF_BOARD if os.path.exists(REF_BOARD) else None
+
+
+def ref_cache_trace(script):
+    """Feeds a script (capacity line, then "i hash winrate" / "l hash" lines) to the
+    reference's NNCache and returns its answers, one line per lookup."""
+    env = dict(os.environ)
+    env.pop("LD_PRELOAD", None)
+    r = subprocess.run([REF_CACHE], input=script, capture_output=True, text=True, env=env,
+                       timeout=600)
+    if r.returncode != 0:
+        raise RuntimeError("ref_cache failed: " + r.stderr[-500:])
+    return r.stdout.splitlines()
+
+
+def ref_board_replay(games):
+    """Replays move lists through the reference's FullBoard.  Returns one dict per game:
+    {"illegal": index} or {"ko", "superko", "score", "stones"[361], "legal"[362]}."""
+    text = "".join("%d %s\n" % (len(g), " ".join(str(int(m)) for m in g)) for g in games)
+    env = dict(os.environ)
+    env.pop("LD_PRELOAD", None)
+    r = subprocess.run([REF_BOARD], input=text, capture_output=True, text=True, env=env,
+                       timeout=600)
+    if r.returncode != 0:
+        raise RuntimeError("ref_board failed: " + r.stderr[-500:])
+    out = []
+    for line in r.stdout.splitlines():
+        f = line.split()
+        if f[0] == "illegal":
+            out.append({"illegal": int(f[1])})
+        else:
+            out.append({"ko": int(f[1]), "superko": f[2] == "1", "score": float(f[3]),
+                        "stones": [int(c) for c in f[4]], "legal": [c == "1" for c in f[5]]})
+    return out
