@@ -121,7 +121,8 @@ int lzhip_reset_stats(lzhip_handle* h);
 /* Head parameters as Network holds them (reference src/Network.h:166-183),
  * after the same preprocessing as src/Network.cpp:351-352,568-576:
  * bn_*_scale = 1/sqrt(var+1e-5), 1x1 conv biases folded into bn_*_mean.
- * ip_pol_w [362][722], ip1_val_w [256][361], ip2_val_w [256]. */
+ * ip_pol_w [362][722], ip1_val_w [256][361], ip2_val_w [256].  The arrays are
+ * copied; call it while no evaluation that uses the heads is in flight. */
 int lzhip_push_heads(lzhip_handle* h, const float* bn_pol_mean, const float* bn_pol_scale,
                      const float* ip_pol_w, const float* ip_pol_b, const float* bn_val_mean,
                      const float* bn_val_scale, const float* ip1_val_w,
