@@ -78,6 +78,17 @@ public:
     virtual int max_concurrency() const { return 1; }
     // in [n][18*361] -> pol [n][722], val [n][361]; throws std::runtime_error.
     virtual void forward_batch(int n, const float* in, float* pol, float* val) = 0;
+    // Input planes that hold only 0 and 1 (what the engine's feature planes are) may be
+    // handed over one bit per value: kInputWords 32-bit words per position, bit
+    // (c*361 + pt) = plane c at point pt.  run_bits does what forward_batch (heads ==
+    // false: out_a = pol planes, out_b = val plane) or evaluate_heads_batch (heads ==
+    // true: out_a = policy, out_b = value) does.  Executors that do not take bits say so.
+    static constexpr int kInputWords = (LZHIP_INPUT_SIZE + 31) / 32;
+    virtual bool accepts_bits() const { return false; }
+    virtual void run_bits(int /*n*/, const uint32_t* /*bits*/, bool /*heads*/,
+                          float /*temperature*/, float* /*out_a*/, float* /*out_b*/) {
+        throw std::logic_error("this executor does not take bit-packed planes");
+    }
     // Whether evaluate_heads_batch can be served (head parameters are on board).
     virtual bool has_heads() const { return false; }
     // Tower + heads for n positions: policy [n][362] (softmax at `temperature`),
@@ -148,6 +159,10 @@ private:
         float* val;   // raw value plane [361], or the value scalar
         bool heads = false;
         float temperature = 1.0f;
+        // the planes one bit per value, filled by the calling thread when every value is
+        // exactly 0 or 1 (then `packed`); 32 times less to gather and to send to the device
+        bool packed = false;
+        uint32_t bits[BatchExecutor::kInputWords];
         std::mutex mu;
         std::condition_variable cv;
         int state = 0;  // 0 pending, 1 done, 2 halted, 3 failed

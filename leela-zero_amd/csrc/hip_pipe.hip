@@ -111,6 +111,8 @@ public:
             sl.dval.alloc(B * kPts);
             sl.dpolicy.alloc(B * 362);
             sl.dvalue.alloc(B);
+            sl.hbits.alloc(B * kInputWords);
+            sl.dbits.alloc(B * kInputWords);
             HIP_CHECK(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
         }
         m_act0.alloc(B * kPts * m_C0p);
@@ -197,7 +199,7 @@ public:
         std::lock_guard<std::mutex> lk(m_mu);
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
-        run_forward(n, d_in, d_pol, d_val);
+        run_forward(n, d_in, nullptr, d_pol, d_val);
         HIP_CHECK(hipGetLastError());
     }
 
@@ -212,7 +214,18 @@ public:
     // the lock, so that the next batch is queued on the device while this one
     // runs and host-side copies overlap device work.
     void forward_batch(int n, const float* in, float* pol, float* val) override {
-        run_host_batch(n, in, false, 1.0f, pol, val);
+        run_host_batch(n, in, nullptr, false, 1.0f, pol, val);
+    }
+
+    // Bit-packed planes: 816 bytes per position travel instead of 26 KB; the first kernel
+    // expands them.  Results are those of the float path on the same 0/1 planes.
+    bool accepts_bits() const override { return true; }
+    void run_bits(int n, const uint32_t* bits, bool heads, float temperature, float* out_a,
+                  float* out_b) override {
+        if (heads && !m_heads_ready) throw std::invalid_argument("push_heads has not been called");
+        if (heads && !(temperature > 0.0f))
+            throw std::invalid_argument("temperature must be positive");
+        run_host_batch(n, nullptr, bits, heads, temperature, out_a, out_b);
     }
 
     // The same path with the heads computed on the device: policy [n][362] and the
@@ -221,11 +234,11 @@ public:
                               float* value) override {
         if (!m_heads_ready) throw std::invalid_argument("push_heads has not been called");
         if (!(temperature > 0.0f)) throw std::invalid_argument("temperature must be positive");
-        run_host_batch(n, in, true, temperature, policy, value);
+        run_host_batch(n, in, nullptr, true, temperature, policy, value);
     }
 
-    void run_host_batch(int n, const float* in, bool heads, float temperature, float* out_a,
-                        float* out_b) {
+    void run_host_batch(int n, const float* in, const uint32_t* bits, bool heads,
+                        float temperature, float* out_a, float* out_b) {
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
         IoSlot* sl = nullptr;
@@ -253,12 +266,23 @@ public:
         } release{this, sl};
         // sizes of the two results per position, staged through hpol / hval
         const size_t na = heads ? 362 : 2 * kPts, nb = heads ? 1 : kPts;
-        std::memcpy(sl->hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
+        if (bits)
+            std::memcpy(sl->hbits.p, bits, sizeof(uint32_t) * (size_t)n * kInputWords);
+        else
+            std::memcpy(sl->hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
         {
             std::lock_guard<std::mutex> lk(m_mu);
-            HIP_CHECK(hipMemcpyAsync(sl->din.p, sl->hin.p, sizeof(float) * (size_t)n * kInPlanes * kPts,
-                                     hipMemcpyHostToDevice, m_stream));
-            run_forward(n, sl->din.p, sl->dpol.p, sl->dval.p);
+            if (bits) {
+                HIP_CHECK(hipMemcpyAsync(sl->dbits.p, sl->hbits.p,
+                                         sizeof(uint32_t) * (size_t)n * kInputWords,
+                                         hipMemcpyHostToDevice, m_stream));
+                run_forward(n, nullptr, sl->dbits.p, sl->dpol.p, sl->dval.p);
+            } else {
+                HIP_CHECK(hipMemcpyAsync(sl->din.p, sl->hin.p,
+                                         sizeof(float) * (size_t)n * kInPlanes * kPts,
+                                         hipMemcpyHostToDevice, m_stream));
+                run_forward(n, sl->din.p, nullptr, sl->dpol.p, sl->dval.p);
+            }
             const float* da = sl->dpol.p;
             const float* db = sl->dval.p;
             if (heads) {
@@ -323,7 +347,7 @@ public:
         HIP_CHECK(hipSetDevice(m_device));
         HIP_CHECK(hipMemcpyAsync(m_din.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts,
                                  hipMemcpyHostToDevice, m_stream));
-        run_forward(n, m_din.p, m_dpol.p, m_dval.p);
+        run_forward(n, m_din.p, nullptr, m_dpol.p, m_dval.p);
         HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
                       m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
         launch_heads(m_dpol.p, m_dval.p, hp, temperature, m_dpolicy.p, m_dlogits.p, m_dvalue.p,
@@ -413,7 +437,7 @@ public:
         if ((int)m_layers.size() * 3 + 2 > kTimerPool)
             throw std::invalid_argument("network too deep for the timer pool");
         m_timer_used = 0;
-        enqueue_forward(n, d_in, d_pol, d_val, true);
+        enqueue_forward(n, d_in, nullptr, d_pol, d_val, true);
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipStreamSynchronize(m_stream));
         for (int k = 0; k < LZHIP_K_COUNT; k++) { ms[k] = 0.0f; launches[k] = 0; }
@@ -481,24 +505,25 @@ private:
     // copies).  On the device the replay measured no faster than stream launches
     // (the gaps between these kernels are drain and cache write-back, not launch
     // latency), so plain stream launches are the default.
-    typedef std::tuple<int, const float*, float*, float*> GraphKey;
+    typedef std::tuple<int, const void*, float*, float*> GraphKey;
     void clear_graphs() {
         for (auto& kv : m_graphs) (void)hipGraphExecDestroy(kv.second);
         m_graphs.clear();
     }
-    void run_forward(int n, const float* d_in, float* d_pol, float* d_val) {
+    // d_in: fp32 planes, or, when null, d_bits: the planes one bit per value
+    void run_forward(int n, const float* d_in, const uint32_t* d_bits, float* d_pol, float* d_val) {
         if (!m_use_graph) {
-            enqueue_forward(n, d_in, d_pol, d_val, false);
+            enqueue_forward(n, d_in, d_bits, d_pol, d_val, false);
             return;
         }
-        const GraphKey key(n, d_in, d_pol, d_val);
+        const GraphKey key(n, d_in ? (const void*)d_in : (const void*)d_bits, d_pol, d_val);
         auto it = m_graphs.find(key);
         if (it == m_graphs.end()) {
             if (m_graphs.size() >= 64) clear_graphs();
             hipGraph_t g = nullptr;
             hipGraphExec_t ge = nullptr;
             HIP_CHECK(hipStreamBeginCapture(m_stream, hipStreamCaptureModeThreadLocal));
-            enqueue_forward(n, d_in, d_pol, d_val, false);
+            enqueue_forward(n, d_in, d_bits, d_pol, d_val, false);
             HIP_CHECK(hipStreamEndCapture(m_stream, &g));
             const hipError_t e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
             (void)hipGraphDestroy(g);
@@ -512,11 +537,16 @@ private:
     // M_l straight into V_{l+1}; the spatial activation is written only where a
     // later layer adds it back as a skip connection (layer 0 and every block
     // output), and by the last layer for the 1x1 heads.
-    void enqueue_forward(int n, const float* d_in, float* d_pol, float* d_val, bool timed) {
+    void enqueue_forward(int n, const float* d_in, const uint32_t* d_bits, float* d_pol,
+                         float* d_val, bool timed) {
         const int nl = (int)m_layers.size();
         const int Tu = n * kTilesPerBoard;
-        launch_pack_input<P>(d_in, m_act0.p, n, kInPlanes, m_C0p, m_stream,
-                             timer(timed, LZHIP_K_PACK));
+        if (d_in)
+            launch_pack_input<P>(d_in, m_act0.p, n, kInPlanes, m_C0p, m_stream,
+                                 timer(timed, LZHIP_K_PACK));
+        else
+            launch_pack_input_bits<P>(d_bits, m_act0.p, n, kInPlanes, m_C0p, m_stream,
+                                      timer(timed, LZHIP_K_PACK));
         launch_in_transform<P>(m_act0.p, m_V.p, n, m_C0p, m_Tp, m_stream,
                                timer(timed, LZHIP_K_IN));
         int cur = 0, nxt = 1;  // block input (skip) / block output
@@ -630,7 +660,9 @@ private:
     // "copied out" at once; their device work is ordered by the one stream.
     struct IoSlot {
         PinnedBuf<float> hin, hpol, hval;
+        PinnedBuf<uint32_t> hbits;
         DevBuf<float> din, dpol, dval, dpolicy, dvalue;
+        DevBuf<uint32_t> dbits;
         hipEvent_t done = nullptr;
         bool busy = false;
     };

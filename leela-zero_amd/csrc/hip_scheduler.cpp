@@ -136,11 +136,33 @@ int HIPScheduler::evaluate_raw(const float* in, float temperature, float* policy
     return submit(req);
 }
 
+// Packs planes that hold only +0.0f and 1.0f, one bit per value; false (and `bits`
+// unspecified) as soon as any other value shows up.
+static bool pack_planes(const float* in, uint32_t* bits) {
+    static_assert(sizeof(float) == sizeof(uint32_t), "float size");
+    constexpr uint32_t kOne = 0x3f800000u;
+    uint32_t word = 0, other = 0;
+    int w = 0;
+    for (int i = 0; i < kInSize; i++) {
+        uint32_t v;
+        std::memcpy(&v, in + i, sizeof(v));
+        other |= (v != 0u && v != kOne) ? 1u : 0u;
+        word |= (uint32_t)(v == kOne) << (i & 31);
+        if ((i & 31) == 31) {
+            bits[w++] = word;
+            word = 0;
+        }
+    }
+    if (kInSize & 31) bits[w] = word;
+    return other == 0;
+}
+
 int HIPScheduler::submit(const std::shared_ptr<Request>& req) {
     if (m_draining.load()) {
         m_halted++;
         return LZHIP_EHALT;
     }
+    req->packed = m_exec && m_exec->accepts_bits() && pack_planes(req->in, req->bits);
     m_outstanding++;
     {
         std::lock_guard<std::mutex> lk(m_mutex);
@@ -192,6 +214,7 @@ int HIPScheduler::submit(const std::shared_ptr<Request>& req) {
 // and decays by one caller per batch.
 void HIPScheduler::worker() {
     std::vector<float> in, pol, val;
+    std::vector<uint32_t> bits((size_t)m_max_batch * BatchExecutor::kInputWords);
     in.resize((size_t)m_max_batch * kInSize);
     pol.resize((size_t)m_max_batch * kPolSize);
     val.resize((size_t)m_max_batch * kValSize);
@@ -258,12 +281,23 @@ void HIPScheduler::worker() {
         }
         if (batch.empty()) continue;
         const int n = (int)batch.size();  // m_inflight was raised under the lock above
-        for (int i = 0; i < n; i++)
-            std::memcpy(in.data() + (size_t)i * kInSize, batch[i]->in, sizeof(float) * kInSize);
+        bool all_packed = true;
+        for (int i = 0; i < n; i++) all_packed = all_packed && batch[i]->packed;
+        if (all_packed) {
+            for (int i = 0; i < n; i++)
+                std::memcpy(bits.data() + (size_t)i * BatchExecutor::kInputWords, batch[i]->bits,
+                            sizeof(uint32_t) * BatchExecutor::kInputWords);
+        } else {
+            for (int i = 0; i < n; i++)
+                std::memcpy(in.data() + (size_t)i * kInSize, batch[i]->in, sizeof(float) * kInSize);
+        }
         int outcome = 1;
         const auto t0 = std::chrono::steady_clock::now();
         try {
-            if (batch[0]->heads)
+            if (all_packed)
+                m_exec->run_bits(n, bits.data(), batch[0]->heads, batch[0]->temperature,
+                                 pol.data(), val.data());
+            else if (batch[0]->heads)
                 m_exec->evaluate_heads_batch(n, in.data(), batch[0]->temperature, pol.data(),
                                              val.data());
             else

@@ -30,6 +30,12 @@ struct LaunchTimer {
 };
 
 // NCHW fp32 planes [n][C][361] -> act [n][361][Cp] (channels >= C zero).
+// 32-bit words of one position's 18 x 361 input planes packed one bit per value.
+constexpr int kInputWords = (18 * 361 + 31) / 32;
+
+template <typename P>
+void launch_pack_input_bits(const uint32_t* bits, P* act, int n, int C, int Cp, hipStream_t s,
+                            LaunchTimer* t);
 template <typename P>
 void launch_pack_input(const float* in, P* act, int n, int C, int Cp, hipStream_t s,
                        LaunchTimer* t);

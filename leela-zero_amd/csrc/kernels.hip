@@ -124,6 +124,35 @@ void launch_pack_input(const float* in, P* act, int n, int C, int Cp, hipStream_
            Cp);
 }
 
+// The same from bit-packed planes: bit (c*361 + pt) of a board's kInputWords words is
+// plane c at point pt (planes that hold only 0 and 1, which is what the engine feeds).
+template <typename P>
+__global__ __launch_bounds__(256) void pack_input_bits_k(const uint32_t* __restrict__ bits,
+                                                         P* __restrict__ act, int n, int C,
+                                                         int Cp) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t total = (size_t)n * kPts * Cp;
+    if (gid >= total) return;
+    const int c = (int)(gid % Cp);
+    const size_t bp = gid / Cp;
+    const int pt = (int)(bp % kPts);
+    const size_t b = bp / kPts;
+    float v = 0.0f;
+    if (c < C) {
+        const int bit = c * kPts + pt;
+        v = (float)((bits[b * kInputWords + (bit >> 5)] >> (bit & 31)) & 1u);
+    }
+    act[gid] = to_storage<P>(v);
+}
+
+template <typename P>
+void launch_pack_input_bits(const uint32_t* bits, P* act, int n, int C, int Cp, hipStream_t s,
+                            LaunchTimer* t) {
+    const size_t total = (size_t)n * kPts * Cp;
+    launch(pack_input_bits_k<P>, dim3((unsigned)((total + 255) / 256)), dim3(256), s, t, bits, act,
+           n, C, Cp);
+}
+
 // ---------------------------------------------------------------------------
 // Winograd input transform V = B^T d B (reference src/CPUPipe.cpp:63-183).
 // One lane owns one tile and ChanVec<P>::N consecutive channels; consecutive
@@ -1613,6 +1642,8 @@ void launch_heads(const float* pol, const float* val, HeadParams hp, float tempe
 #define INSTANTIATE(P)                                                                         \
     template void launch_pack_input<P>(const float*, P*, int, int, int, hipStream_t,           \
                                        LaunchTimer*);                                          \
+    template void launch_pack_input_bits<P>(const uint32_t*, P*, int, int, int, hipStream_t,   \
+                                            LaunchTimer*);                                     \
     template void launch_in_transform<P>(const P*, P*, int, int, int, hipStream_t,             \
                                          LaunchTimer*);                                        \
     template void launch_gemm<P>(const P*, const P*, P*, int, int, int, int, hipStream_t,      \

@@ -9,6 +9,9 @@
 //   * an executor failure reaches the caller as an exception;
 //   * with an executor that accepts two batches at a time, two batches are in
 //     flight together and all of the above still holds;
+//   * planes that hold only 0 and 1 reach an executor that takes bits one bit per
+//     value, any other value sends the whole batch down the float path, and both give
+//     each caller the result of its own planes;
 //   * a steady population of callers smaller than max_batch ends up in one
 //     batch per round instead of two alternating partial ones.
 #include <atomic>
@@ -71,6 +74,76 @@ public:
 private:
     int m_mb, m_delay, m_conc;
 };
+
+// Takes bit-packed planes; the answer depends on every input value:
+// pol[i] = sum_k (k % 7 + 1) * x[k] + i, val[i] = x[i] (first 361 values).
+class BitsExec : public BatchExecutor {
+public:
+    explicit BitsExec(int mb) : m_mb(mb) {}
+    int max_batch() const override { return m_mb; }
+    int max_concurrency() const override { return 2; }
+    bool accepts_bits() const override { return true; }
+    static float digest(const float* x) {
+        double s = 0.0;
+        for (int k = 0; k < LZHIP_INPUT_SIZE; k++) s += (double)(k % 7 + 1) * x[k];
+        return (float)s;
+    }
+    void forward_batch(int n, const float* in, float* pol, float* val) override {
+        std::this_thread::sleep_for(std::chrono::microseconds(100));
+        for (int b = 0; b < n; b++) {
+            const float* x = in + (size_t)b * LZHIP_INPUT_SIZE;
+            const float d = digest(x);
+            for (int i = 0; i < LZHIP_POL_SIZE; i++) pol[(size_t)b * LZHIP_POL_SIZE + i] = d + i;
+            for (int i = 0; i < LZHIP_VAL_SIZE; i++) val[(size_t)b * LZHIP_VAL_SIZE + i] = x[i];
+        }
+        float_batches++;
+    }
+    void run_bits(int n, const uint32_t* bits, bool heads, float, float* a, float* b) override {
+        CHECK(!heads);
+        std::vector<float> in((size_t)n * LZHIP_INPUT_SIZE);
+        for (int p = 0; p < n; p++)
+            for (int k = 0; k < LZHIP_INPUT_SIZE; k++)
+                in[(size_t)p * LZHIP_INPUT_SIZE + k] =
+                    (float)((bits[(size_t)p * kInputWords + (k >> 5)] >> (k & 31)) & 1u);
+        forward_batch(n, in.data(), a, b);
+        float_batches--;
+        bit_batches++;
+    }
+    std::atomic<int> float_batches{0}, bit_batches{0};
+private:
+    int m_mb;
+};
+
+static void test_bit_packed_requests() {
+    auto* be = new BitsExec(8);
+    HIPScheduler s{std::unique_ptr<BatchExecutor>(be)};
+    std::atomic<int> ok{0};
+    std::vector<std::thread> th;
+    for (int t = 0; t < 10; t++)
+        th.emplace_back([&, t] {
+            std::vector<float> in(LZHIP_INPUT_SIZE), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
+            uint64_t st = 1234567 + 977 * t;
+            for (int r = 0; r < 30; r++) {
+                for (auto& v : in) {
+                    st = st * 6364136223846793005ull + 1442695040888963407ull;
+                    v = (st >> 62) == 0 ? 1.0f : 0.0f;
+                }
+                in[LZHIP_INPUT_SIZE - 1] = 1.0f;                 // the last, partial word
+                if (t == 3 && r % 4 == 0) in[100 + r] = 0.5f;    // not a 0/1 plane
+                if (t == 5 && r % 7 == 0) in[7] = -0.0f;         // nor is a negative zero
+                s.forward(in, pol, val);
+                const float d = BitsExec::digest(in.data());
+                for (int i = 0; i < LZHIP_POL_SIZE; i++) CHECK(pol[i] == d + i);
+                for (int i = 0; i < LZHIP_VAL_SIZE; i++) CHECK(val[i] == in[i]);
+                ok++;
+            }
+        });
+    for (auto& t : th) t.join();
+    CHECK(ok == 300);
+    CHECK(be->bit_batches > 0 && be->float_batches > 0);
+    std::printf("bit-packed: %d batches as bits, %d as floats\n", be->bit_batches.load(),
+                be->float_batches.load());
+}
 
 static void one_call(HIPScheduler& s, float a, float b, std::atomic<int>& ok,
                      std::atomic<int>& halted) {
@@ -209,6 +282,7 @@ int main() {
     test_concurrent(48, 8, 20);
     test_concurrent(48, 8, 20, 2);  // two batches in flight
     test_concurrent(5, 8, 20, 2);
+    test_bit_packed_requests();
     test_population_batches(1);
     test_population_batches(2);
     for (int c = 1; c <= 2; c++) {

@@ -377,3 +377,24 @@ def test_other_widths(pkg, netgen, orc, precision, filters, batch):
     x = netgen.synthetic_inputs(batch, seed=filters)
     check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=[0, batch - 1])
     pipe.close()
+
+
+def test_bit_packed_and_float_requests_agree(pkg, netgen, orc):
+    """Queued requests whose planes hold only 0 and 1 travel one bit per value; any other
+    value sends the request down the float path.  Both must give bit-for-bit what the
+    batch executor gives for the same planes handed over as floats."""
+    print("case: bit-packed requests", flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 2, 64, 91, pkg.FP32, 4)
+    x = netgen.synthetic_inputs(4, seed=12)
+    x[1, 3, 17] = 0.25          # not a 0/1 plane
+    x[2, 16, :] = 1.0
+    x[3, 17, 360] = 1.0         # the very last value: the partial last word
+    pol, val = pipe.forward_batch(x)
+    for i in range(4):
+        p1, v1 = pipe.forward(x[i])
+        assert np.array_equal(p1, pol[i]) and np.array_equal(v1, val[i]), i
+    policy, value, _ = pipe.evaluate_batch(x)
+    for i in (0, 1, 3):
+        pe, ve = pipe.forward_eval(x[i])
+        assert np.abs(pe - policy[i]).max() <= 1e-6 and abs(ve - value[i]) <= 1e-6, i
+    pipe.close()
