@@ -109,10 +109,7 @@ public:
             sl.din.alloc(B * kInPlanes * kPts);
             sl.dpol.alloc(B * 2 * kPts);
             sl.dval.alloc(B * kPts);
-            sl.dpolicy.alloc(B * 362);
-            sl.dvalue.alloc(B);
             sl.hbits.alloc(B * kInputWords);
-            sl.dbits.alloc(B * kInputWords);
             HIP_CHECK(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
         }
         m_act0.alloc(B * kPts * m_C0p);
@@ -264,7 +261,7 @@ public:
                 self->m_slot_cv.notify_all();
             }
         } release{this, sl};
-        // sizes of the two results per position, staged through hpol / hval
+        // sizes of the two results per position, both written by the device into hpol / hval
         const size_t na = heads ? 362 : 2 * kPts, nb = heads ? 1 : kPts;
         if (bits)
             std::memcpy(sl->hbits.p, bits, sizeof(uint32_t) * (size_t)n * kInputWords);
@@ -272,32 +269,28 @@ public:
             std::memcpy(sl->hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
         {
             std::lock_guard<std::mutex> lk(m_mu);
+            // Pinned host memory is mapped into the device's address space: the first
+            // kernel reads the packed planes and the last ones write the results straight
+            // through it, so that no copy command sits between this batch's kernels and
+            // the next batch's (each one is a bubble of tens of microseconds on the
+            // stream).  Float planes, 32 times larger, still go by copy.
+            float* out_a_dev = heads ? sl->dpol.p : sl->hpol.p;   // raw planes: straight to host
+            float* out_b_dev = heads ? sl->dval.p : sl->hval.p;
             if (bits) {
-                HIP_CHECK(hipMemcpyAsync(sl->dbits.p, sl->hbits.p,
-                                         sizeof(uint32_t) * (size_t)n * kInputWords,
-                                         hipMemcpyHostToDevice, m_stream));
-                run_forward(n, nullptr, sl->dbits.p, sl->dpol.p, sl->dval.p);
+                run_forward(n, nullptr, sl->hbits.p, out_a_dev, out_b_dev);
             } else {
                 HIP_CHECK(hipMemcpyAsync(sl->din.p, sl->hin.p,
                                          sizeof(float) * (size_t)n * kInPlanes * kPts,
                                          hipMemcpyHostToDevice, m_stream));
-                run_forward(n, sl->din.p, nullptr, sl->dpol.p, sl->dval.p);
+                run_forward(n, sl->din.p, nullptr, out_a_dev, out_b_dev);
             }
-            const float* da = sl->dpol.p;
-            const float* db = sl->dval.p;
             if (heads) {
                 HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
                               m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
-                launch_heads(sl->dpol.p, sl->dval.p, hp, temperature, sl->dpolicy.p, nullptr,
-                             sl->dvalue.p, n, m_stream);
-                da = sl->dpolicy.p;
-                db = sl->dvalue.p;
+                launch_heads(sl->dpol.p, sl->dval.p, hp, temperature, sl->hpol.p, nullptr,
+                             sl->hval.p, n, m_stream);
             }
             HIP_CHECK(hipGetLastError());
-            HIP_CHECK(hipMemcpyAsync(sl->hpol.p, da, sizeof(float) * (size_t)n * na,
-                                     hipMemcpyDeviceToHost, m_stream));
-            HIP_CHECK(hipMemcpyAsync(sl->hval.p, db, sizeof(float) * (size_t)n * nb,
-                                     hipMemcpyDeviceToHost, m_stream));
             HIP_CHECK(hipEventRecord(sl->done, m_stream));
         }
         HIP_CHECK(hipEventSynchronize(sl->done));
@@ -661,8 +654,7 @@ private:
     struct IoSlot {
         PinnedBuf<float> hin, hpol, hval;
         PinnedBuf<uint32_t> hbits;
-        DevBuf<float> din, dpol, dval, dpolicy, dvalue;
-        DevBuf<uint32_t> dbits;
+        DevBuf<float> din, dpol, dval;
         hipEvent_t done = nullptr;
         bool busy = false;
     };
