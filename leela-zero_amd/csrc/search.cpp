@@ -313,6 +313,7 @@ UCTSearch::~UCTSearch() {
     }
     m_pool_cv.notify_all();
     for (auto& th : m_pool) th.join();
+    if (m_reaper.joinable()) m_reaper.join();
     free_tree(m_root);
 }
 
@@ -623,8 +624,11 @@ void UCTSearch::advance(int move) {
             }
         }
     }
-    free_tree(m_root);
+    // The discarded part of the tree is freed while the next search is already running.
+    if (m_reaper.joinable()) m_reaper.join();
+    Node* old = m_root;
     m_root = keep;
+    if (old) m_reaper = std::thread([old] { free_tree(old); });
 }
 
 // ---------------------------------------------------------------------------

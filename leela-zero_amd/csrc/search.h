@@ -193,6 +193,7 @@ private:
     int m_active = 0;
     bool m_quit = false;
     const go::Position* m_root_pos = nullptr;
+    std::thread m_reaper;   // frees the part of the tree a move left behind
 };
 
 // Plays cfg.moves moves of self-play from the empty board; fills `out` and, if
