@@ -93,8 +93,9 @@ int lzhip_forward(lzhip_handle* h, const float* in, float* pol, float* val);
 
 /* Batch executor under the scheduler: OpenCL_Network::forward(batch)
  * (reference src/OpenCL.cpp:142-329).  n <= max_batch positions, host
- * buffers, blocking (H2D + tower + 1x1 heads + D2H).  Serialised internally;
- * does not go through the request queue. */
+ * buffers, blocking (H2D + tower + 1x1 heads + D2H).  Thread-safe: as many
+ * callers as the handle has lanes are served side by side, further ones
+ * wait.  Does not go through the request queue. */
 int lzhip_forward_batch(lzhip_handle* h, int n, const float* in, float* pol, float* val);
 
 /* Same executor on buffers that already live in device memory (the reference
@@ -103,8 +104,20 @@ int lzhip_forward_batch(lzhip_handle* h, int n, const float* in, float* pol, flo
  * handle's stream and returns without waiting; lzhip_sync waits. */
 int lzhip_forward_batch_device(lzhip_handle* h, int n, const void* d_in, void* d_pol,
                                void* d_val);
+/* The handle owns lzhip_lanes(h) lanes: a stream each, with the working buffers of
+ * one forward, as each batch worker of the reference owns an OpenCLContext with its
+ * command queue and buffers (src/OpenCL.h:64-84, src/OpenCLScheduler.cpp:113-130,
+ * :291).  Forwards enqueued on different lanes run side by side on the device, and
+ * since a chain of dependent kernels leaves the device partly idle at every kernel
+ * boundary, two batches on two lanes finish sooner than the same two on one.
+ * lzhip_forward_batch_device is lane 0; lzhip_forward_batch and the request queue
+ * use one lane per batch in flight. */
+int lzhip_lanes(lzhip_handle* h);
+int lzhip_forward_batch_device_lane(lzhip_handle* h, int lane, int n, const void* d_in,
+                                    void* d_pol, void* d_val);
+/* Waits for the work enqueued on every lane. */
 int lzhip_sync(lzhip_handle* h);
-/* The hipStream_t the handle launches on (for callers that record events). */
+/* The hipStream_t of lane 0 (for callers that record events). */
 void* lzhip_stream(lzhip_handle* h);
 
 /* ForwardPipe::drain / resume (reference src/ForwardPipe.h:69-70,

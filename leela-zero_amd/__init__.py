@@ -35,7 +35,8 @@ KERNEL_CLASSES = ["pack_input", "in_transform", "gemm", "out_transform", "head_c
 # Every symbol include/lzhip.h declares.
 EXPORTS = [
     "lzhip_create", "lzhip_destroy", "lzhip_push_weights", "lzhip_forward",
-    "lzhip_forward_batch", "lzhip_forward_batch_device", "lzhip_sync", "lzhip_stream",
+    "lzhip_forward_batch", "lzhip_forward_batch_device", "lzhip_lanes",
+    "lzhip_forward_batch_device_lane", "lzhip_sync", "lzhip_stream",
     "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats", "lzhip_push_heads",
     "lzhip_evaluate_batch", "lzhip_forward_eval", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
     "lzhip_debug_layer", "lzhip_get_act_scales", "lzhip_profile_forward", "lzhip_last_error",
@@ -136,6 +137,9 @@ def lib():
         L.lzhip_forward.argtypes = [ctypes.c_void_p, _fp, _fp, _fp]
         L.lzhip_forward_batch.argtypes = [ctypes.c_void_p, ctypes.c_int, _fp, _fp, _fp]
         L.lzhip_forward_batch_device.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 3
+        L.lzhip_lanes.argtypes = [ctypes.c_void_p]
+        L.lzhip_forward_batch_device_lane.argtypes = ([ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
+                                                      + [ctypes.c_void_p] * 3)
         L.lzhip_sync.argtypes = [ctypes.c_void_p]
         L.lzhip_drain.argtypes = [ctypes.c_void_p]
         L.lzhip_resume.argtypes = [ctypes.c_void_p]
@@ -354,10 +358,17 @@ class HIPScheduler:
         _check(lib().lzhip_forward_batch(self._h, n, _ptr(x), _ptr(pol), _ptr(val)))
         return pol, val
 
-    def forward_batch_device(self, n, d_in, d_pol, d_val):
-        """Asynchronous forward on device pointers (ints); see sync()."""
+    def lanes(self):
+        """Number of lanes (streams with their own working buffers) of the handle."""
         self._need()
-        _check(lib().lzhip_forward_batch_device(self._h, int(n), d_in, d_pol, d_val))
+        return lib().lzhip_lanes(self._h)
+
+    def forward_batch_device(self, n, d_in, d_pol, d_val, lane=0):
+        """Asynchronous forward on device pointers (ints) on one lane; see sync().
+        Forwards on different lanes run side by side and need buffers of their own."""
+        self._need()
+        _check(lib().lzhip_forward_batch_device_lane(self._h, int(lane), int(n), d_in, d_pol,
+                                                     d_val))
 
     def sync(self):
         self._need()

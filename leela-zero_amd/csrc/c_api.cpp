@@ -111,8 +111,20 @@ int lzhip_forward_batch_device(lzhip_handle* h, int n, const void* d_in, void* d
                                void* d_val) {
     if (!h || !d_in || !d_pol || !d_val) return fail(LZHIP_EINVAL, "null argument");
     GUARD_BEGIN
-    h->pipe->forward_device(n, static_cast<const float*>(d_in), static_cast<float*>(d_pol),
+    h->pipe->forward_device(0, n, static_cast<const float*>(d_in), static_cast<float*>(d_pol),
                             static_cast<float*>(d_val));
+    return LZHIP_OK;
+    GUARD_END
+}
+
+int lzhip_lanes(lzhip_handle* h) { return h ? h->pipe->lanes() : 0; }
+
+int lzhip_forward_batch_device_lane(lzhip_handle* h, int lane, int n, const void* d_in,
+                                    void* d_pol, void* d_val) {
+    if (!h || !d_in || !d_pol || !d_val) return fail(LZHIP_EINVAL, "null argument");
+    GUARD_BEGIN
+    h->pipe->forward_device(lane, n, static_cast<const float*>(d_in),
+                            static_cast<float*>(d_pol), static_cast<float*>(d_val));
     return LZHIP_OK;
     GUARD_END
 }

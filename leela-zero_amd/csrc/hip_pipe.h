@@ -23,8 +23,12 @@ public:
     virtual void push_weights(int n_layers, const float* const* U, const float* const* bn_mean,
                               const float* const* bn_scale, const float* pol_w,
                               const float* val_w) = 0;
-    // Asynchronous forward on device-resident buffers (fp32 in/out).
-    virtual void forward_device(int n, const float* d_in, float* d_pol, float* d_val) = 0;
+    // Asynchronous forward on device-resident buffers (fp32 in/out), enqueued on one of
+    // the pipe's lanes (a stream with its own working buffers); forwards on different
+    // lanes run side by side.  sync() waits for every lane; stream() is lane 0's.
+    virtual int lanes() const = 0;
+    virtual void forward_device(int lane, int n, const float* d_in, float* d_pol,
+                                float* d_val) = 0;
     virtual void sync() = 0;
     virtual void* stream() = 0;
 

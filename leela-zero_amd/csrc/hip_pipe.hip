@@ -86,7 +86,7 @@ public:
         if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
             throw std::runtime_error(std::string("device is ") + prop.gcnArchName +
                                      ", this library contains gfx950 code only");
-        HIP_CHECK(hipStreamCreate(&m_stream));
+        for (auto& ln : m_lane) HIP_CHECK(hipStreamCreate(&ln.stream));
         m_Fp = round_up(filters, 64);
         if (!gemm_supports_channels<P>(m_Fp))
             throw std::invalid_argument(
@@ -112,10 +112,12 @@ public:
             sl.hbits.alloc(B * kInputWords);
             HIP_CHECK(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
         }
-        m_act0.alloc(B * kPts * m_C0p);
-        for (auto& a : m_act) a.alloc(B * kPts * m_Fp);
-        m_V.alloc((size_t)kPos * m_Tp * m_Fp);
-        m_M.alloc((size_t)kPos * m_Tp * m_Fp);
+        for (auto& ln : m_lane) {
+            ln.act0.alloc(B * kPts * m_C0p);
+            for (auto& a : ln.act) a.alloc(B * kPts * m_Fp);
+            ln.V.alloc((size_t)kPos * m_Tp * m_Fp);
+            ln.M.alloc((size_t)kPos * m_Tp * m_Fp);
+        }
         m_scalar.alloc(4);
         for (int i = 0; i < kTimerPool; i++) {
             HIP_CHECK(hipEventCreate(&m_ev_start[i]));
@@ -125,7 +127,8 @@ public:
 
     ~HIPPipeImpl() override {
         (void)hipSetDevice(m_device);
-        if (m_stream) (void)hipStreamSynchronize(m_stream);
+        for (auto& ln : m_lane)
+            if (ln.stream) (void)hipStreamSynchronize(ln.stream);
         clear_graphs();
         for (int i = 0; i < kTimerPool; i++) {
             if (m_ev_start[i]) (void)hipEventDestroy(m_ev_start[i]);
@@ -133,7 +136,8 @@ public:
         }
         for (auto& sl : m_slot)
             if (sl.done) (void)hipEventDestroy(sl.done);
-        if (m_stream) (void)hipStreamDestroy(m_stream);
+        for (auto& ln : m_lane)
+            if (ln.stream) (void)hipStreamDestroy(ln.stream);
     }
 
     int max_batch() const override { return m_max_batch; }
@@ -141,14 +145,16 @@ public:
     bool has_heads() const override { return m_heads_ready; }
     int filters() const override { return m_filters; }
     int precision() const override { return precision_of<P>(); }
-    void* stream() override { return m_stream; }
+    void* stream() override { return m_lane[0].stream; }
+    int lanes() const override { return kLanes; }
     std::vector<float> act_scales() const override { return m_s; }
 
     // -------------------------------------------------------------------
     void push_weights(int n_layers, const float* const* U, const float* const* bn_mean,
                       const float* const* bn_scale, const float* pol_w,
                       const float* val_w) override {
-        std::lock_guard<std::mutex> lk(m_mu);
+        Lane& ln = m_lane[0];
+        std::lock_guard<std::mutex> lk(ln.mu);
         if (n_layers < 1 || (n_layers % 2) != 1)
             throw std::invalid_argument("n_layers must be 1 + 2*blocks");
         if (!m_layers.empty()) throw std::invalid_argument("push_weights called twice");
@@ -188,21 +194,23 @@ public:
         m_s.assign(n_layers + 1, 1.0f);
         for (int l = 0; l < n_layers; l++) upload_bn(l);
         if (precision_of<P>() == LZHIP_FP16) calibrate();
-        HIP_CHECK(hipStreamSynchronize(m_stream));
+        HIP_CHECK(hipStreamSynchronize(ln.stream));
     }
 
     // -------------------------------------------------------------------
-    void forward_device(int n, const float* d_in, float* d_pol, float* d_val) override {
-        std::lock_guard<std::mutex> lk(m_mu);
+    void forward_device(int lane, int n, const float* d_in, float* d_pol, float* d_val) override {
+        if (lane < 0 || lane >= kLanes) throw std::invalid_argument("no such lane");
+        Lane& ln = m_lane[lane];
+        std::lock_guard<std::mutex> lk(ln.mu);
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
-        run_forward(n, d_in, nullptr, d_pol, d_val);
+        run_forward(ln, n, d_in, nullptr, d_pol, d_val);
         HIP_CHECK(hipGetLastError());
     }
 
     void sync() override {
         HIP_CHECK(hipSetDevice(m_device));
-        HIP_CHECK(hipStreamSynchronize(m_stream));
+        for (auto& ln : m_lane) HIP_CHECK(hipStreamSynchronize(ln.stream));
     }
 
     // Host-buffer forward.  Up to kIoSlots callers may be inside at once: each
@@ -268,7 +276,9 @@ public:
         else
             std::memcpy(sl->hin.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts);
         {
-            std::lock_guard<std::mutex> lk(m_mu);
+            // each staging slot has a lane of its own: two batches run side by side
+            Lane& ln = m_lane[sl - m_slot];
+            std::lock_guard<std::mutex> lk(ln.mu);
             // Pinned host memory is mapped into the device's address space: the first
             // kernel reads the packed planes and the last ones write the results straight
             // through it, so that no copy command sits between this batch's kernels and
@@ -277,21 +287,21 @@ public:
             float* out_a_dev = heads ? sl->dpol.p : sl->hpol.p;   // raw planes: straight to host
             float* out_b_dev = heads ? sl->dval.p : sl->hval.p;
             if (bits) {
-                run_forward(n, nullptr, sl->hbits.p, out_a_dev, out_b_dev);
+                run_forward(ln, n, nullptr, sl->hbits.p, out_a_dev, out_b_dev);
             } else {
                 HIP_CHECK(hipMemcpyAsync(sl->din.p, sl->hin.p,
                                          sizeof(float) * (size_t)n * kInPlanes * kPts,
-                                         hipMemcpyHostToDevice, m_stream));
-                run_forward(n, sl->din.p, nullptr, out_a_dev, out_b_dev);
+                                         hipMemcpyHostToDevice, ln.stream));
+                run_forward(ln, n, sl->din.p, nullptr, out_a_dev, out_b_dev);
             }
             if (heads) {
                 HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
                               m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
                 launch_heads(sl->dpol.p, sl->dval.p, hp, temperature, sl->hpol.p, nullptr,
-                             sl->hval.p, n, m_stream);
+                             sl->hval.p, n, ln.stream);
             }
             HIP_CHECK(hipGetLastError());
-            HIP_CHECK(hipEventRecord(sl->done, m_stream));
+            HIP_CHECK(hipEventRecord(sl->done, ln.stream));
         }
         HIP_CHECK(hipEventSynchronize(sl->done));
         std::memcpy(out_a, sl->hpol.p, sizeof(float) * (size_t)n * na);
@@ -300,7 +310,8 @@ public:
 
     // -------------------------------------------------------------------
     void push_heads(const HeadWeightsHost& hw) override {
-        std::lock_guard<std::mutex> lk(m_mu);
+        Lane& ln = m_lane[0];
+        std::lock_guard<std::mutex> lk(ln.mu);
         HIP_CHECK(hipSetDevice(m_device));
         auto up = [&](DevBuf<float>& d, const float* src, size_t n) {
             d.alloc(n);
@@ -333,20 +344,21 @@ public:
 
     void evaluate_batch(int n, const float* in, float temperature, float* policy, float* value,
                         float* logits, float* pol, float* val) override {
-        std::lock_guard<std::mutex> lk(m_mu);
+        Lane& ln = m_lane[0];
+        std::lock_guard<std::mutex> lk(ln.mu);
         check_ready(n);
         if (!m_heads_ready) throw std::invalid_argument("push_heads has not been called");
         if (!(temperature > 0.0f)) throw std::invalid_argument("temperature must be positive");
         HIP_CHECK(hipSetDevice(m_device));
         HIP_CHECK(hipMemcpyAsync(m_din.p, in, sizeof(float) * (size_t)n * kInPlanes * kPts,
-                                 hipMemcpyHostToDevice, m_stream));
-        run_forward(n, m_din.p, nullptr, m_dpol.p, m_dval.p);
+                                 hipMemcpyHostToDevice, ln.stream));
+        run_forward(ln, n, m_din.p, nullptr, m_dpol.p, m_dval.p);
         HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
                       m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
         launch_heads(m_dpol.p, m_dval.p, hp, temperature, m_dpolicy.p, m_dlogits.p, m_dvalue.p,
-                     n, m_stream);
+                     n, ln.stream);
         HIP_CHECK(hipGetLastError());
-        HIP_CHECK(hipStreamSynchronize(m_stream));
+        HIP_CHECK(hipStreamSynchronize(ln.stream));
         HIP_CHECK(hipMemcpy(policy, m_dpolicy.p, sizeof(float) * (size_t)n * 362, hipMemcpyDeviceToHost));
         HIP_CHECK(hipMemcpy(value, m_dvalue.p, sizeof(float) * (size_t)n, hipMemcpyDeviceToHost));
         if (logits)
@@ -360,7 +372,8 @@ public:
     // -------------------------------------------------------------------
     void debug_layer(int layer, int n, const float* act_in, const float* res, float* Vout,
                      float* Mout, float* Yout) override {
-        std::lock_guard<std::mutex> lk(m_mu);
+        Lane& ln = m_lane[0];
+        std::lock_guard<std::mutex> lk(ln.mu);
         check_ready(n);
         if (layer < 0 || layer >= (int)m_layers.size()) throw std::invalid_argument("bad layer");
         HIP_CHECK(hipSetDevice(m_device));
@@ -371,30 +384,30 @@ public:
         DevBuf<float> d_planes, d_res, d_sc, d_mn;
         d_planes.alloc((size_t)n * C * kPts);
         HIP_CHECK(hipMemcpy(d_planes.p, act_in, sizeof(float) * (size_t)n * C * kPts, hipMemcpyHostToDevice));
-        P* a_in = (layer == 0) ? m_act0.p : m_act[0].p;
-        launch_pack_input<P>(d_planes.p, a_in, n, C, Cp, m_stream, nullptr);
+        P* a_in = (layer == 0) ? ln.act0.p : ln.act[0].p;
+        launch_pack_input<P>(d_planes.p, a_in, n, C, Cp, ln.stream, nullptr);
         const P* r = nullptr;
         if (res) {
             d_res.alloc((size_t)n * F * kPts);
             HIP_CHECK(hipMemcpy(d_res.p, res, sizeof(float) * (size_t)n * F * kPts, hipMemcpyHostToDevice));
-            launch_pack_input<P>(d_res.p, m_act[1].p, n, F, m_Fp, m_stream, nullptr);
-            r = m_act[1].p;
+            launch_pack_input<P>(d_res.p, ln.act[1].p, n, F, m_Fp, ln.stream, nullptr);
+            r = ln.act[1].p;
         }
         std::vector<float> sc(m_Fp, 0.0f), mn(m_Fp, 0.0f);
         for (int k = 0; k < F; k++) { sc[k] = L.scale[k]; mn[k] = L.mean[k]; }
         d_sc.alloc(m_Fp); d_mn.alloc(m_Fp);
         HIP_CHECK(hipMemcpy(d_sc.p, sc.data(), sizeof(float) * m_Fp, hipMemcpyHostToDevice));
         HIP_CHECK(hipMemcpy(d_mn.p, mn.data(), sizeof(float) * m_Fp, hipMemcpyHostToDevice));
-        launch_in_transform<P>(a_in, m_V.p, n, Cp, m_Tp, m_stream, nullptr);
-        launch_gemm<P>(m_V.p, L.U.p, m_M.p, Tu, m_Tp, Cp, m_Fp, m_stream, nullptr);
-        launch_out_transform<P>(m_M.p, r, m_act[2].p, d_sc.p, d_mn.p, 1.0f, n, m_Fp, m_Tp,
-                                m_stream, nullptr);
+        launch_in_transform<P>(a_in, ln.V.p, n, Cp, m_Tp, ln.stream, nullptr);
+        launch_gemm<P>(ln.V.p, L.U.p, ln.M.p, Tu, m_Tp, Cp, m_Fp, ln.stream, nullptr);
+        launch_out_transform<P>(ln.M.p, r, ln.act[2].p, d_sc.p, d_mn.p, 1.0f, n, m_Fp, m_Tp,
+                                ln.stream, nullptr);
         HIP_CHECK(hipGetLastError());
-        HIP_CHECK(hipStreamSynchronize(m_stream));
+        HIP_CHECK(hipStreamSynchronize(ln.stream));
         const int T = n * kTilesPerBoard;
         if (Vout) {
             std::vector<P> h((size_t)kPos * m_Tp * Cp);
-            HIP_CHECK(hipMemcpy(h.data(), m_V.p, h.size() * sizeof(P), hipMemcpyDeviceToHost));
+            HIP_CHECK(hipMemcpy(h.data(), ln.V.p, h.size() * sizeof(P), hipMemcpyDeviceToHost));
             for (int t = 0; t < T; t++)
                 for (int p = 0; p < kPos; p++)
                     for (int c = 0; c < C; c++)
@@ -403,7 +416,7 @@ public:
         }
         if (Mout) {
             std::vector<P> h((size_t)kPos * m_Tp * m_Fp);
-            HIP_CHECK(hipMemcpy(h.data(), m_M.p, h.size() * sizeof(P), hipMemcpyDeviceToHost));
+            HIP_CHECK(hipMemcpy(h.data(), ln.M.p, h.size() * sizeof(P), hipMemcpyDeviceToHost));
             for (int t = 0; t < T; t++)
                 for (int p = 0; p < kPos; p++)
                     for (int k = 0; k < F; k++)
@@ -412,7 +425,7 @@ public:
         }
         if (Yout) {
             std::vector<P> h((size_t)n * kPts * m_Fp);
-            HIP_CHECK(hipMemcpy(h.data(), m_act[2].p, h.size() * sizeof(P), hipMemcpyDeviceToHost));
+            HIP_CHECK(hipMemcpy(h.data(), ln.act[2].p, h.size() * sizeof(P), hipMemcpyDeviceToHost));
             for (int b = 0; b < n; b++)
                 for (int pt = 0; pt < kPts; pt++)
                     for (int k = 0; k < F; k++)
@@ -424,15 +437,16 @@ public:
     // -------------------------------------------------------------------
     void profile_forward(int n, const float* d_in, float* d_pol, float* d_val, float* ms,
                          int* launches) override {
-        std::lock_guard<std::mutex> lk(m_mu);
+        Lane& ln = m_lane[0];
+        std::lock_guard<std::mutex> lk(ln.mu);
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
         if ((int)m_layers.size() * 3 + 2 > kTimerPool)
             throw std::invalid_argument("network too deep for the timer pool");
         m_timer_used = 0;
-        enqueue_forward(n, d_in, nullptr, d_pol, d_val, true);
+        enqueue_forward(ln, n, d_in, nullptr, d_pol, d_val, true);
         HIP_CHECK(hipGetLastError());
-        HIP_CHECK(hipStreamSynchronize(m_stream));
+        HIP_CHECK(hipStreamSynchronize(ln.stream));
         for (int k = 0; k < LZHIP_K_COUNT; k++) { ms[k] = 0.0f; launches[k] = 0; }
         for (int i = 0; i < m_timer_used; i++) {
             float t = 0.0f;
@@ -443,6 +457,19 @@ public:
     }
 
 private:
+    typedef std::tuple<int, const void*, float*, float*> GraphKey;
+    // A lane is a stream with the working buffers of one forward.  Two batches on two
+    // lanes run side by side on the device: each kernel's start-up and tail overlap with
+    // the other lane's work, which a single chain of dependent kernels cannot do.
+    // Lane 0 also serves calibration, profiling and the single-batch entry points.
+    struct Lane {
+        hipStream_t stream = nullptr;
+        std::mutex mu;  // serialises enqueues on this lane
+        DevBuf<P> act0, act[3], V, M;
+        std::map<GraphKey, hipGraphExec_t> graphs;
+    };
+    static constexpr int kLanes = 2;
+
     struct Layer {
         int C = 0, Cp = 0;
         DevBuf<P> U;
@@ -482,14 +509,14 @@ private:
     }
 
     // Activation buffer roles rotate: cur = block input, mid, nxt = block output.
-    void run_conv(int l, int n, const P* in, const P* res, P* out, bool timed) {
+    void run_conv(Lane& ln, int l, int n, const P* in, const P* res, P* out, bool timed) {
         Layer& L = m_layers[l];
         const int Tu = n * kTilesPerBoard;
-        launch_in_transform<P>(in, m_V.p, n, L.Cp, m_Tp, m_stream, timer(timed, LZHIP_K_IN));
-        launch_gemm<P>(m_V.p, L.U.p, m_M.p, Tu, m_Tp, L.Cp, m_Fp, m_stream,
+        launch_in_transform<P>(in, ln.V.p, n, L.Cp, m_Tp, ln.stream, timer(timed, LZHIP_K_IN));
+        launch_gemm<P>(ln.V.p, L.U.p, ln.M.p, Tu, m_Tp, L.Cp, m_Fp, ln.stream,
                        timer(timed, LZHIP_K_GEMM));
-        launch_out_transform<P>(m_M.p, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, m_Tp,
-                                m_stream, timer(timed, LZHIP_K_OUT));
+        launch_out_transform<P>(ln.M.p, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, m_Tp,
+                                ln.stream, timer(timed, LZHIP_K_OUT));
     }
 
     // With LZHIP_GRAPH=1 the 165 launches of a forward are captured once per
@@ -498,78 +525,82 @@ private:
     // copies).  On the device the replay measured no faster than stream launches
     // (the gaps between these kernels are drain and cache write-back, not launch
     // latency), so plain stream launches are the default.
-    typedef std::tuple<int, const void*, float*, float*> GraphKey;
+    void clear_graphs(Lane& ln) {
+        for (auto& kv : ln.graphs) (void)hipGraphExecDestroy(kv.second);
+        ln.graphs.clear();
+    }
     void clear_graphs() {
-        for (auto& kv : m_graphs) (void)hipGraphExecDestroy(kv.second);
-        m_graphs.clear();
+        for (auto& ln : m_lane) clear_graphs(ln);
     }
     // d_in: fp32 planes, or, when null, d_bits: the planes one bit per value
-    void run_forward(int n, const float* d_in, const uint32_t* d_bits, float* d_pol, float* d_val) {
+    void run_forward(Lane& ln, int n, const float* d_in, const uint32_t* d_bits, float* d_pol,
+                     float* d_val) {
         if (!m_use_graph) {
-            enqueue_forward(n, d_in, d_bits, d_pol, d_val, false);
+            enqueue_forward(ln, n, d_in, d_bits, d_pol, d_val, false);
             return;
         }
         const GraphKey key(n, d_in ? (const void*)d_in : (const void*)d_bits, d_pol, d_val);
-        auto it = m_graphs.find(key);
-        if (it == m_graphs.end()) {
-            if (m_graphs.size() >= 64) clear_graphs();
+        auto it = ln.graphs.find(key);
+        if (it == ln.graphs.end()) {
+            if (ln.graphs.size() >= 64) clear_graphs(ln);
             hipGraph_t g = nullptr;
             hipGraphExec_t ge = nullptr;
-            HIP_CHECK(hipStreamBeginCapture(m_stream, hipStreamCaptureModeThreadLocal));
-            enqueue_forward(n, d_in, d_bits, d_pol, d_val, false);
-            HIP_CHECK(hipStreamEndCapture(m_stream, &g));
+            HIP_CHECK(hipStreamBeginCapture(ln.stream, hipStreamCaptureModeThreadLocal));
+            enqueue_forward(ln, n, d_in, d_bits, d_pol, d_val, false);
+            HIP_CHECK(hipStreamEndCapture(ln.stream, &g));
             const hipError_t e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
             (void)hipGraphDestroy(g);
             HIP_CHECK(e);
-            it = m_graphs.emplace(key, ge).first;
+            it = ln.graphs.emplace(key, ge).first;
         }
-        HIP_CHECK(hipGraphLaunch(it->second, m_stream));
+        HIP_CHECK(hipGraphLaunch(it->second, ln.stream));
     }
 
     // Layer loop.  Every layer but the last ends in the fused kernel that turns
     // M_l straight into V_{l+1}; the spatial activation is written only where a
     // later layer adds it back as a skip connection (layer 0 and every block
     // output), and by the last layer for the 1x1 heads.
-    void enqueue_forward(int n, const float* d_in, const uint32_t* d_bits, float* d_pol,
-                         float* d_val, bool timed) {
+    void enqueue_forward(Lane& ln, int n, const float* d_in, const uint32_t* d_bits,
+                         float* d_pol, float* d_val, bool timed) {
         const int nl = (int)m_layers.size();
         const int Tu = n * kTilesPerBoard;
         if (d_in)
-            launch_pack_input<P>(d_in, m_act0.p, n, kInPlanes, m_C0p, m_stream,
+            launch_pack_input<P>(d_in, ln.act0.p, n, kInPlanes, m_C0p, ln.stream,
                                  timer(timed, LZHIP_K_PACK));
         else
-            launch_pack_input_bits<P>(d_bits, m_act0.p, n, kInPlanes, m_C0p, m_stream,
+            launch_pack_input_bits<P>(d_bits, ln.act0.p, n, kInPlanes, m_C0p, ln.stream,
                                       timer(timed, LZHIP_K_PACK));
-        launch_in_transform<P>(m_act0.p, m_V.p, n, m_C0p, m_Tp, m_stream,
+        launch_in_transform<P>(ln.act0.p, ln.V.p, n, m_C0p, m_Tp, ln.stream,
                                timer(timed, LZHIP_K_IN));
         int cur = 0, nxt = 1;  // block input (skip) / block output
         for (int l = 0; l < nl; l++) {
             Layer& L = m_layers[l];
-            launch_gemm<P>(m_V.p, L.U.p, m_M.p, Tu, m_Tp, L.Cp, m_Fp, m_stream,
+            launch_gemm<P>(ln.V.p, L.U.p, ln.M.p, Tu, m_Tp, L.Cp, m_Fp, ln.stream,
                            timer(timed, LZHIP_K_GEMM));
             const bool block_end = (l % 2) == 0;      // layer 0 and second convs
-            const P* res = (block_end && l >= 2) ? m_act[cur].p : nullptr;
-            P* out = l == 0 ? m_act[cur].p : m_act[nxt].p;
+            const P* res = (block_end && l >= 2) ? ln.act[cur].p : nullptr;
+            P* out = l == 0 ? ln.act[cur].p : ln.act[nxt].p;
             if (l == nl - 1) {
-                launch_out_transform<P>(m_M.p, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n,
-                                        m_Fp, m_Tp, m_stream, timer(timed, LZHIP_K_OUT));
-                launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, m_stream,
+                launch_out_transform<P>(ln.M.p, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n,
+                                        m_Fp, m_Tp, ln.stream, timer(timed, LZHIP_K_OUT));
+                launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, ln.stream,
                                     timer(timed, LZHIP_K_HEAD));
             } else {
-                launch_out_in_transform<P>(m_M.p, res, block_end ? out : nullptr, m_V.p,
+                launch_out_in_transform<P>(ln.M.p, res, block_end ? out : nullptr, ln.V.p,
                                            L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, m_Tp,
-                                           m_stream, timer(timed, LZHIP_K_OUTIN));
+                                           ln.stream, timer(timed, LZHIP_K_OUTIN));
             }
             if (block_end && l >= 2) { const int o = cur; cur = nxt; nxt = o; }
         }
     }
 
     float absmax(const P* x, size_t count) {
-        HIP_CHECK(hipMemsetAsync(m_scalar.p, 0, sizeof(float), m_stream));
-        launch_absmax<P>(x, count, m_scalar.p, m_stream);
+        Lane& ln = m_lane[0];
+        HIP_CHECK(hipMemsetAsync(m_scalar.p, 0, sizeof(float), ln.stream));
+        launch_absmax<P>(x, count, m_scalar.p, ln.stream);
         float v = 0.0f;
-        HIP_CHECK(hipMemcpyAsync(&v, m_scalar.p, sizeof(float), hipMemcpyDeviceToHost, m_stream));
-        HIP_CHECK(hipStreamSynchronize(m_stream));
+        HIP_CHECK(hipMemcpyAsync(&v, m_scalar.p, sizeof(float), hipMemcpyDeviceToHost, ln.stream));
+        HIP_CHECK(hipStreamSynchronize(ln.stream));
         return v;
     }
 
@@ -582,6 +613,7 @@ private:
     // exact in real arithmetic.  Trained networks keep |x| small and get
     // s_l = 1 (plain fp16 storage, as the reference's half pipeline).
     void calibrate() {
+        Lane& ln = m_lane[0];
         const int n = m_max_batch < 8 ? m_max_batch : 8;
         std::vector<float> in((size_t)n * kInPlanes * kPts, 0.0f);
         uint64_t st = 0x9E3779B97F4A7C15ull;
@@ -600,7 +632,7 @@ private:
             for (int pt = 0; pt < kPts; pt++) x[16 * kPts + pt] = 1.0f;
         }
         HIP_CHECK(hipMemcpy(m_din.p, in.data(), in.size() * sizeof(float), hipMemcpyHostToDevice));
-        launch_pack_input<P>(m_din.p, m_act0.p, n, kInPlanes, m_C0p, m_stream, nullptr);
+        launch_pack_input<P>(m_din.p, ln.act0.p, n, kInPlanes, m_C0p, ln.stream, nullptr);
 
         const float target = 16.0f;
         const int nl = (int)m_layers.size();
@@ -613,11 +645,11 @@ private:
             for (int attempt = 0; attempt < 8; attempt++) {
                 upload_bn(l);
                 if (attempt == 0) {
-                    run_conv(l, n, src, res, dst, false);
+                    run_conv(ln, l, n, src, res, dst, false);
                 } else {
                     Layer& L = m_layers[l];
-                    launch_out_transform<P>(m_M.p, res, dst, L.d_scale.p, L.d_mean.p, L.rfac, n,
-                                            m_Fp, m_Tp, m_stream, nullptr);
+                    launch_out_transform<P>(ln.M.p, res, dst, L.d_scale.p, L.d_mean.p, L.rfac, n,
+                                            m_Fp, m_Tp, ln.stream, nullptr);
                 }
                 const float mx = absmax(dst, cnt);
                 if (!(mx < 60000.0f)) {  // saturated (or NaN): coarser scale, try again
@@ -635,10 +667,10 @@ private:
             }
             throw std::runtime_error("activation-scale calibration did not converge");
         };
-        settle(0, m_act0.p, nullptr, m_act[cur].p);
+        settle(0, ln.act0.p, nullptr, ln.act[cur].p);
         for (int l = 1; l + 1 < nl; l += 2) {
-            settle(l, m_act[cur].p, nullptr, m_act[mid].p);
-            settle(l + 1, m_act[mid].p, m_act[cur].p, m_act[nxt].p);
+            settle(l, ln.act[cur].p, nullptr, ln.act[mid].p);
+            settle(l + 1, ln.act[mid].p, ln.act[cur].p, ln.act[nxt].p);
             const int o = cur; cur = nxt; nxt = o;
         }
     }
@@ -646,11 +678,10 @@ private:
     static constexpr int kTimerPool = 512;
     int m_device, m_max_batch, m_filters;
     int m_Fp = 0, m_C0p = 0, m_Tp = 0;
-    hipStream_t m_stream = nullptr;
-    std::mutex m_mu;
+    Lane m_lane[kLanes];
     DevBuf<float> m_din, m_dpol, m_dval, m_w3, m_scalar;  // evaluate_batch / calibration
     // Staging of forward_batch: kIoSlots batches may be between "copied in" and
-    // "copied out" at once; their device work is ordered by the one stream.
+    // "copied out" at once, slot i on lane i.
     struct IoSlot {
         PinnedBuf<float> hin, hpol, hval;
         PinnedBuf<uint32_t> hbits;
@@ -658,11 +689,10 @@ private:
         hipEvent_t done = nullptr;
         bool busy = false;
     };
-    static constexpr int kIoSlots = 2;
+    static constexpr int kIoSlots = kLanes;
     IoSlot m_slot[kIoSlots];
     std::mutex m_slot_mu;
     std::condition_variable m_slot_cv;
-    DevBuf<P> m_act0, m_act[3], m_V, m_M;
     std::vector<Layer> m_layers;
     std::vector<float> m_s;  // activation scales, m_s[0] = input
     DevBuf<float> m_h[10], m_dpolicy, m_dlogits, m_dvalue;
@@ -671,7 +701,6 @@ private:
     int m_timer_class[kTimerPool] = {};
     int m_timer_used = 0;
     LaunchTimer m_timer;
-    std::map<GraphKey, hipGraphExec_t> m_graphs;
     bool m_use_graph = std::getenv("LZHIP_GRAPH") != nullptr;
 };
 

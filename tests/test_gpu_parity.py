@@ -276,6 +276,64 @@ def test_device_resident_forward_and_profile(pkg, netgen, orc):
     pipe.close()
 
 
+def test_lanes_run_side_by_side_with_equal_results(pkg, netgen, orc):
+    """Forwards of different batches enqueued on the handle's two lanes, many in a row with no
+    synchronisation between them, give bit for bit what each batch gives alone on lane 0;
+    host-buffer calls from two threads (one lane each) likewise.  A lane that does not
+    exist is refused."""
+    import threading
+    import torch
+    print("case: lanes", flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 128, 81, pkg.FP16, 16)
+    assert pipe.lanes() == 2
+    xa = netgen.synthetic_inputs(16, seed=21)
+    xb = netgen.synthetic_inputs(11, seed=22)
+    want_a = pipe.forward_batch(xa)
+    want_b = pipe.forward_batch(xb)
+    d_a, d_b = torch.from_numpy(xa).cuda(), torch.from_numpy(xb).cuda()
+    pol = [torch.zeros(16, 722, device="cuda") for _ in range(2)]
+    val = [torch.zeros(16, 361, device="cuda") for _ in range(2)]
+    torch.cuda.synchronize()
+    for rep in range(6):
+        pipe.forward_batch_device(16, d_a.data_ptr(), pol[0].data_ptr(), val[0].data_ptr(), lane=0)
+        pipe.forward_batch_device(11, d_b.data_ptr(), pol[1].data_ptr(), val[1].data_ptr(), lane=1)
+    pipe.sync()
+    assert np.array_equal(pol[0].cpu().numpy(), want_a[0])
+    assert np.array_equal(val[0].cpu().numpy(), want_a[1])
+    assert np.array_equal(pol[1].cpu().numpy()[:11], want_b[0])
+    assert np.array_equal(val[1].cpu().numpy()[:11], want_b[1])
+    # the roles swapped: lane 1 takes the batch lane 0 had
+    pipe.forward_batch_device(16, d_a.data_ptr(), pol[1].data_ptr(), val[1].data_ptr(), lane=1)
+    pipe.forward_batch_device(11, d_b.data_ptr(), pol[0].data_ptr(), val[0].data_ptr(), lane=0)
+    pipe.sync()
+    assert np.array_equal(pol[1].cpu().numpy(), want_a[0])
+    assert np.array_equal(pol[0].cpu().numpy()[:11], want_b[0])
+    for lane in (2, -1):
+        with pytest.raises(ValueError):
+            pipe.forward_batch_device(4, d_a.data_ptr(), pol[0].data_ptr(), val[0].data_ptr(),
+                                      lane=lane)
+
+    bad = []
+    def caller(x, want):
+        for _ in range(8):
+            got = pipe.forward_batch(x)
+            if not (np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])):
+                bad.append(1)
+    th = [threading.Thread(target=caller, args=(xa, want_a)),
+          threading.Thread(target=caller, args=(xb, want_b)),
+          threading.Thread(target=caller, args=(xa[:5], (want_a[0][:5], want_a[1][:5])))]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert not bad
+    # against the oracle as well, so that "equal" is not "equally wrong"
+    for i in (0, 10):
+        rp, rv = ref.forward(xb[i])
+        assert rel_l2(want_b[0][i], rp) <= 2e-2 and rel_l2(want_b[1][i], rv) <= 2e-2
+    pipe.close()
+
+
 def test_graph_replays_match_stream_launches(pkg, netgen, orc):
     """The forward is replayed from a captured HIP graph.  Replays of several graphs
     (different batch sizes and buffers), with other work and synchronisations in between,
