@@ -256,6 +256,21 @@ def main():
     for _ in range(host_steps):
         pipe.forward_batch(x)
     host_dt = (time.perf_counter() - t0) / host_steps
+    # ... and from as many threads as the handle has lanes, a batch each at a time
+    host2_dt = None
+    if lanes > 1:
+        import threading
+
+        def host_caller():
+            for _ in range(host_steps):
+                pipe.forward_batch(x)
+        th = [threading.Thread(target=host_caller) for _ in range(lanes)]
+        t0 = time.perf_counter()
+        for t in th:
+            t.start()
+        for t in th:
+            t.join()
+        host2_dt = (time.perf_counter() - t0) / (host_steps * lanes)
 
     # per-kernel-class device time, measured live with HIP events on the pipe's stream
     ms = np.zeros(pkg.K_COUNT)
@@ -336,7 +351,9 @@ def main():
         "gemm_mfma_util_pct": 100.0 * gemm_rate / peak,
         "host_buffers": {"value": B / host_dt, "unit": "evals/s", "ms_per_step": host_dt * 1e3,
                          "note": "lzhip_forward_batch on pageable host arrays, sequential calls "
-                                 "(PCIe and staging copies inside the timed region)"},
+                                 "(PCIe and staging copies inside the timed region)",
+                         "callers_as_lanes": (None if host2_dt is None else
+                                              {"value": B / host2_dt, "callers": lanes})},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
