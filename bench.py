@@ -162,8 +162,9 @@ def main():
     ap.add_argument("--precision", choices=["fp16", "fp32"], default="fp16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-reps", type=int, default=5)
-    ap.add_argument("--lanes", type=int, default=2,
-                    help="forward workload: batches kept on the device side by side (1 or 2)")
+    ap.add_argument("--lanes", type=int, default=0,
+                    help="forward workload: batches kept on the device side by side; 0 = as "
+                         "many as the handle has (2, or 3 up to batch 32)")
     ap.add_argument("--workload", choices=["forward", "search"], default="forward",
                     help="forward: the headline metric; search: BASELINE configs[4]")
     ap.add_argument("--threads", type=int, default=16, help="search threads (search workload)")
@@ -214,7 +215,7 @@ def main():
     nl = net.n_layers
 
     d_in = torch.from_numpy(x).cuda()
-    lanes = max(1, min(args.lanes, pipe.lanes()))
+    lanes = pipe.lanes() if args.lanes <= 0 else max(1, min(args.lanes, pipe.lanes()))
     d_pols = [torch.zeros(B, 722, device="cuda") for _ in range(lanes)]
     d_vals = [torch.zeros(B, 361, device="cuda") for _ in range(lanes)]
     d_pol, d_val = d_pols[0], d_vals[0]

@@ -86,7 +86,10 @@ public:
         if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
             throw std::runtime_error(std::string("device is ") + prop.gcnArchName +
                                      ", this library contains gfx950 code only");
-        for (auto& ln : m_lane) HIP_CHECK(hipStreamCreate(&ln.stream));
+        // Small batches leave more of the device idle at every kernel boundary: a third
+        // lane pays up to batch 32 (+10 %) and no longer at 64 (-2 %).
+        m_n_lanes = max_batch <= 32 ? 3 : 2;
+        for (int i = 0; i < m_n_lanes; i++) HIP_CHECK(hipStreamCreate(&m_lane[i].stream));
         m_Fp = round_up(filters, 64);
         if (!gemm_supports_channels<P>(m_Fp))
             throw std::invalid_argument(
@@ -102,7 +105,8 @@ public:
         m_din.alloc(B * kInPlanes * kPts);
         m_dpol.alloc(B * 2 * kPts);
         m_dval.alloc(B * kPts);
-        for (auto& sl : m_slot) {
+        for (int i = 0; i < m_n_lanes; i++) {
+            IoSlot& sl = m_slot[i];
             sl.hin.alloc(B * kInPlanes * kPts);
             sl.hpol.alloc(B * 2 * kPts);
             sl.hval.alloc(B * kPts);
@@ -112,7 +116,8 @@ public:
             sl.hbits.alloc(B * kInputWords);
             HIP_CHECK(hipEventCreateWithFlags(&sl.done, hipEventDisableTiming));
         }
-        for (auto& ln : m_lane) {
+        for (int i = 0; i < m_n_lanes; i++) {
+            Lane& ln = m_lane[i];
             ln.act0.alloc(B * kPts * m_C0p);
             for (auto& a : ln.act) a.alloc(B * kPts * m_Fp);
             ln.V.alloc((size_t)kPos * m_Tp * m_Fp);
@@ -141,12 +146,12 @@ public:
     }
 
     int max_batch() const override { return m_max_batch; }
-    int max_concurrency() const override { return kIoSlots; }
+    int max_concurrency() const override { return m_n_lanes; }
     bool has_heads() const override { return m_heads_ready; }
     int filters() const override { return m_filters; }
     int precision() const override { return precision_of<P>(); }
     void* stream() override { return m_lane[0].stream; }
-    int lanes() const override { return kLanes; }
+    int lanes() const override { return m_n_lanes; }
     std::vector<float> act_scales() const override { return m_s; }
 
     // -------------------------------------------------------------------
@@ -199,7 +204,7 @@ public:
 
     // -------------------------------------------------------------------
     void forward_device(int lane, int n, const float* d_in, float* d_pol, float* d_val) override {
-        if (lane < 0 || lane >= kLanes) throw std::invalid_argument("no such lane");
+        if (lane < 0 || lane >= m_n_lanes) throw std::invalid_argument("no such lane");
         Lane& ln = m_lane[lane];
         std::lock_guard<std::mutex> lk(ln.mu);
         check_ready(n);
@@ -210,7 +215,7 @@ public:
 
     void sync() override {
         HIP_CHECK(hipSetDevice(m_device));
-        for (auto& ln : m_lane) HIP_CHECK(hipStreamSynchronize(ln.stream));
+        for (int i = 0; i < m_n_lanes; i++) HIP_CHECK(hipStreamSynchronize(m_lane[i].stream));
     }
 
     // Host-buffer forward.  Up to kIoSlots callers may be inside at once: each
@@ -250,12 +255,12 @@ public:
         {
             std::unique_lock<std::mutex> lk(m_slot_mu);
             m_slot_cv.wait(lk, [&] {
-                for (auto& c : m_slot)
-                    if (!c.busy) return true;
+                for (int i = 0; i < m_n_lanes; i++)
+                    if (!m_slot[i].busy) return true;
                 return false;
             });
-            for (auto& c : m_slot)
-                if (!c.busy) { sl = &c; break; }
+            for (int i = 0; i < m_n_lanes && !sl; i++)
+                if (!m_slot[i].busy) sl = &m_slot[i];
             sl->busy = true;
         }
         struct Release {
@@ -468,7 +473,7 @@ private:
         DevBuf<P> act0, act[3], V, M;
         std::map<GraphKey, hipGraphExec_t> graphs;
     };
-    static constexpr int kLanes = 2;
+    static constexpr int kLanes = 3;   // upper bound; m_n_lanes are in use
 
     struct Layer {
         int C = 0, Cp = 0;
@@ -679,6 +684,7 @@ private:
     int m_device, m_max_batch, m_filters;
     int m_Fp = 0, m_C0p = 0, m_Tp = 0;
     Lane m_lane[kLanes];
+    int m_n_lanes = 2;
     DevBuf<float> m_din, m_dpol, m_dval, m_w3, m_scalar;  // evaluate_batch / calibration
     // Staging of forward_batch: kIoSlots batches may be between "copied in" and
     // "copied out" at once, slot i on lane i.

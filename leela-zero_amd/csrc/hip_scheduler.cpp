@@ -59,10 +59,9 @@ void HIPScheduler::start_worker() {
     std::lock_guard<std::mutex> lk(m_mutex);
     if (m_running) return;
     m_running = true;
-    // Two workers when the executor can hold two batches: one assembles and
-    // submits the next batch while the other waits for the device and hands
-    // results back.
-    const int n = std::max(1, std::min(2, m_exec->max_concurrency()));
+    // As many workers as the executor runs batches side by side: while one waits for the
+    // device and hands results back, the others assemble and submit the next batches.
+    const int n = std::max(1, std::min(3, m_exec->max_concurrency()));
     for (int i = 0; i < n; i++) m_workers.emplace_back(&HIPScheduler::worker, this);
 }
 

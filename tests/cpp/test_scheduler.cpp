@@ -7,7 +7,7 @@
 //     resume() needs an empty queue and re-opens the pipe;
 //   * destruction with idle and with blocked callers ends cleanly;
 //   * an executor failure reaches the caller as an exception;
-//   * with an executor that accepts two batches at a time, two batches are in
+//   * with an executor that accepts two or three batches at a time, that many are in
 //     flight together and all of the above still holds;
 //   * planes that hold only 0 and 1 reach an executor that takes bits one bit per
 //     value, any other value sends the whole batch down the float path, and both give
@@ -179,7 +179,7 @@ static void test_concurrent(int threads, int mb, int reps, int concurrency = 1) 
     CHECK(st.batches == (uint64_t)fe->calls.load());
     if (threads >= 2 * mb) CHECK(st.batches < (uint64_t)threads * reps);  // it did batch
     CHECK(fe->max_inside <= concurrency);
-    if (concurrency == 2 && threads >= 4 * mb) CHECK(fe->max_inside == 2);  // batches overlapped
+    if (concurrency >= 2 && threads >= 4 * mb) CHECK(fe->max_inside == concurrency);  // batches overlapped
     std::printf("concurrent threads=%d mb=%d: %llu batches for %llu requests, max %u\n", threads,
                 mb, (unsigned long long)st.batches, (unsigned long long)st.requests,
                 st.max_batch_seen);
@@ -282,10 +282,13 @@ int main() {
     test_concurrent(48, 8, 20);
     test_concurrent(48, 8, 20, 2);  // two batches in flight
     test_concurrent(5, 8, 20, 2);
+    test_concurrent(48, 8, 20, 3);  // three
+    test_concurrent(9, 8, 20, 3);
     test_bit_packed_requests();
     test_population_batches(1);
     test_population_batches(2);
-    for (int c = 1; c <= 2; c++) {
+    test_population_batches(3);
+    for (int c = 1; c <= 3; c++) {
         test_drain_resume(c);
         test_destroy_with_waiters(c);
         test_executor_failure(c);

@@ -279,13 +279,13 @@ def test_device_resident_forward_and_profile(pkg, netgen, orc):
 def test_lanes_run_side_by_side_with_equal_results(pkg, netgen, orc):
     """Forwards of different batches enqueued on the handle's two lanes, many in a row with no
     synchronisation between them, give bit for bit what each batch gives alone on lane 0;
-    host-buffer calls from two threads (one lane each) likewise.  A lane that does not
+    host-buffer calls from four threads (more than there are lanes) likewise.  A lane that does not
     exist is refused."""
     import threading
     import torch
     print("case: lanes", flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 128, 81, pkg.FP16, 16)
-    assert pipe.lanes() == 2
+    assert pipe.lanes() == 3      # up to batch 32; two above
     xa = netgen.synthetic_inputs(16, seed=21)
     xb = netgen.synthetic_inputs(11, seed=22)
     want_a = pipe.forward_batch(xa)
@@ -308,7 +308,15 @@ def test_lanes_run_side_by_side_with_equal_results(pkg, netgen, orc):
     pipe.sync()
     assert np.array_equal(pol[1].cpu().numpy(), want_a[0])
     assert np.array_equal(pol[0].cpu().numpy()[:11], want_b[0])
-    for lane in (2, -1):
+    # the third lane, alone and beside the others
+    for rep in range(3):
+        pipe.forward_batch_device(11, d_b.data_ptr(), pol[0].data_ptr(), val[0].data_ptr(), lane=0)
+        pipe.forward_batch_device(16, d_a.data_ptr(), pol[1].data_ptr(), val[1].data_ptr(), lane=2)
+    pipe.sync()
+    assert np.array_equal(pol[1].cpu().numpy(), want_a[0])
+    assert np.array_equal(val[1].cpu().numpy(), want_a[1])
+    assert np.array_equal(pol[0].cpu().numpy()[:11], want_b[0])
+    for lane in (3, -1):
         with pytest.raises(ValueError):
             pipe.forward_batch_device(4, d_a.data_ptr(), pol[0].data_ptr(), val[0].data_ptr(),
                                       lane=lane)
@@ -321,7 +329,8 @@ def test_lanes_run_side_by_side_with_equal_results(pkg, netgen, orc):
                 bad.append(1)
     th = [threading.Thread(target=caller, args=(xa, want_a)),
           threading.Thread(target=caller, args=(xb, want_b)),
-          threading.Thread(target=caller, args=(xa[:5], (want_a[0][:5], want_a[1][:5])))]
+          threading.Thread(target=caller, args=(xa[:5], (want_a[0][:5], want_a[1][:5]))),
+          threading.Thread(target=caller, args=(xb[:2], (want_b[0][:2], want_b[1][:2])))]
     for t in th:
         t.start()
     for t in th:
@@ -331,6 +340,9 @@ def test_lanes_run_side_by_side_with_equal_results(pkg, netgen, orc):
     for i in (0, 10):
         rp, rv = ref.forward(xb[i])
         assert rel_l2(want_b[0][i], rp) <= 2e-2 and rel_l2(want_b[1][i], rv) <= 2e-2
+    pipe.close()
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, 64, 82, pkg.FP16, 40)
+    assert pipe.lanes() == 2
     pipe.close()
 
 
