@@ -356,6 +356,8 @@ def main():
                          "callers_as_lanes": (None if host2_dt is None else
                                               {"value": B / host2_dt, "callers": lanes})},
         "cpu_baseline": cpu,
+        "environment": {"device": torch.cuda.get_device_name(0), "hip": torch.version.hip,
+                        "torch": torch.__version__},
     }
     print(json.dumps(out))
 
