@@ -639,11 +639,12 @@ template <typename P>
 void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
                              const float* bn_mean, float rfac, int n, int Kp, int Tp,
                              hipStream_t s, LaunchTimer* t) {
-    // Enough (board, 64-channel) items to occupy most compute units: wide runs; otherwise
-    // spread (measured at 256 filters: 64 channels wins from batch 48, 32 from batch 8 to
-    // 32, 16 at batch 1).
+    // 32 channels per work-group for as long as those work-groups fit the 256 compute units
+    // in one go (a board's arithmetic then spreads over twice as many units), 64 beyond
+    // that (measured at 256 filters: 32 wins up to batch 32, 64 from batch 33, by 6 %); 16 only
+    // for the smallest batches (a wash between batch 6 and 12, a loss at 8 and 16).
     const int items64 = n * (Kp / 64);
-    if (items64 >= 160)
+    if (items64 > 128)
         launch(out_in_transform_k<P, 64>, dim3(items64), dim3(fuse_waves(64) * 64), s, t, M, res,
                act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
     else if (items64 >= 24)
@@ -712,10 +713,17 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
                                                    int tiles_n, int seg) {
     constexpr int EPC = 16 / sizeof(P);   // elements per 16-byte chunk
     constexpr int BK = 128 / sizeof(P);   // contraction extent of one LDS stage
-    constexpr int ROW = BK + EPC;         // padded LDS row, in elements (144 bytes)
+    // LDS rows: padded to 144 bytes, or (the 64-column tile) bare 128-byte rows whose
+    // 16-byte chunks are permuted by the row number, which is just as conflict free for
+    // the fragment reads (16 lanes = 16 rows: 8 chunk slots x 2 row parities = all 64
+    // banks) and brings a stage pair under a third of the LDS, so that three
+    // work-groups share a compute unit instead of two.
+    constexpr bool SWZ = BN == 64 && sizeof(P) == 2;   // fp32 is bound by the matrix pipe: no gain
+    constexpr int ROW = SWZ ? BK : BK + EPC;
     constexpr int WM = BM / 2, WN = BN / 2;
     constexpr int MB = WM / 32, NB = WN / 32;
     constexpr int A_CH = BM * 8 / 256, B_CH = BN * 8 / 256;  // chunks per thread and stage
+    auto slot = [](int row, int chunk) { return SWZ ? (chunk ^ ((row >> 1) & 7)) : chunk; };
     constexpr int CROW = BN + EPC;        // padded row of the staged output tile
     constexpr int STAGE = (BM + BN) * ROW;
     constexpr int SMEM = (2 * STAGE > BM * CROW) ? 2 * STAGE : BM * CROW;
@@ -766,10 +774,10 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
         P* Bs = As + BM * ROW;
 #pragma unroll
         for (int i = 0; i < A_CH; i++)
-            *reinterpret_cast<int4v*>(&As[(lrow + i * 32) * ROW + lch * EPC]) = ra[st][i];
+            *reinterpret_cast<int4v*>(&As[(lrow + i * 32) * ROW + slot(lrow, lch) * EPC]) = ra[st][i];
 #pragma unroll
         for (int i = 0; i < B_CH; i++)
-            *reinterpret_cast<int4v*>(&Bs[(lrow + i * 32) * ROW + lch * EPC]) = rb[st][i];
+            *reinterpret_cast<int4v*>(&Bs[(lrow + i * 32) * ROW + slot(lrow, lch) * EPC]) = rb[st][i];
     };
 
     // NK = Cp / BK is a template argument: the pipeline below is straight-line
@@ -781,7 +789,7 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
     lstore(0, 0);
     __syncthreads();
 
-    const int frow = lane & 31, fk = (lane >> 5) * EPC;
+    const int frow = lane & 31, fk = lane >> 5;   // tile offsets are multiples of 32 rows
 #pragma unroll
     for (int k = 0; k < NK; k++) {
         const int h = k & 1;
@@ -797,11 +805,11 @@ __global__ __launch_bounds__(256) void wino_gemm_k(const P* __restrict__ V,
 #pragma unroll
             for (int i = 0; i < MB; i++)
                 fa[i] = *reinterpret_cast<const int4v*>(
-                    &As[(wy * WM + i * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+                    &As[(wy * WM + i * 32 + frow) * ROW + slot(frow, kc * 2 + fk) * EPC]);
 #pragma unroll
             for (int j = 0; j < NB; j++)
                 fb[j] = *reinterpret_cast<const int4v*>(
-                    &Bs[(wx * WN + j * 32 + frow) * ROW + kc * 2 * EPC + fk]);
+                    &Bs[(wx * WN + j * 32 + frow) * ROW + slot(frow, kc * 2 + fk) * EPC]);
 #pragma unroll
             for (int i = 0; i < MB; i++)
 #pragma unroll
@@ -1409,10 +1417,12 @@ void launch_gemm(const P* V, const P* U, P* M, int T, int Tp, int Cp, int Kp, hi
         }
     }
     const int tiles_m = (T + kGemmBM - 1) / kGemmBM;
-    // 128 x 128 tiles once there are more of them than two per compute unit can hold at a
-    // time; below that the narrower tile gives the chip twice as many independent pieces
-    // (measured at 256 filters: faster up to batch 16, slower from batch 32).
-    if (Kp % 128 == 0 && kPos * tiles_m * (Kp / 128) > 320)
+    // Below the 256 x 256 tile, fp16: the 128 x 64 tile, three work-groups to a compute unit,
+    // gives the chip the most independent pieces (measured at 256 filters: ahead of 128 x 128
+    // tiles, two to a unit, at every batch up to 40, by 4 % at 21 and 1 % at 40); 128 x 128
+    // tiles take over where that would be more than two rounds of the narrow ones.  fp32 (two
+    // narrow work-groups to a unit): 128 x 128 once there are more than 320 of them.
+    if (Kp % 128 == 0 && kPos * tiles_m * (Kp / 128) > (sizeof(P) == 2 ? 600 : 320))
         launch_gemm_bn<P, 128>(V, U, M, tiles_m, Tp, Cp, Kp, s, t);
     else
         launch_gemm_bn<P, 64>(V, U, M, tiles_m, Tp, Cp, Kp, s, t);
