@@ -1406,9 +1406,11 @@ void launch_gemm(const P* V, const P* U, P* M, int T, int Tp, int Cp, int Kp, hi
                  LaunchTimer* t) {
     constexpr int BK = 128 / (int)sizeof(P);
     const int nk = Cp / BK;
-    // The 256 x 256 tile pays off once its tiles can occupy most of the 256 compute units.
+    // The 256 x 256 tile pays off once its tiles can occupy most of the 256 compute units
+    // (measured at 256 filters: from 6 row tiles = 216 work-groups, batch 52; with 5 = 180 the
+    // 128 x 128 tiles are 2 % ahead; fp32 keeps the earlier hand-over at 160).
     const int big_rows = (T + 255) / 256;
-    if (Kp % 256 == 0 && big_rows * (Kp / 256) * kPos >= 160) {
+    if (Kp % 256 == 0 && big_rows * (Kp / 256) * kPos >= (sizeof(P) == 2 ? 200 : 160)) {
         switch (nk) {
 #define LZ_BIG(N) case N: launch_gemm_big<P, N>(V, U, M, T, big_rows, Tp, Cp, Kp, s, t); return;
             LZ_BIG(1) LZ_BIG(2) LZ_BIG(4) LZ_BIG(8) LZ_BIG(16)
