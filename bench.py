@@ -282,6 +282,19 @@ def main():
         cnt += c
     ms /= args.profile_reps
     cnt /= args.profile_reps
+    # the same event-timed forward on lane 0 while another lane works through forwards of
+    # its own: what a launch takes when it shares the device, as in the timed steps above
+    ms2 = None
+    if lanes > 1:
+        ms2 = np.zeros(pkg.K_COUNT)
+        for _ in range(args.profile_reps):
+            for _ in range(3):
+                pipe.forward_batch_device(B, d_in.data_ptr(), d_pols[1].data_ptr(),
+                                          d_vals[1].data_ptr(), lane=1)
+            m, _c = pipe.profile_forward(B, *ptrs)
+            pipe.sync()
+            ms2 += m
+        ms2 /= args.profile_reps
     e = 2 if prec == pkg.FP16 else 4
     gf = gemm_flops(B, F, nl)
     in_b, out_b, fused_b = transform_bytes(B, F, nl, e)
@@ -297,6 +310,14 @@ def main():
         "launches_per_forward": int(cnt[pkg.K_GEMM]),
         "flops_per_launch": gf / cnt[pkg.K_GEMM],
     }
+    roofline["launch_context"] = ("launches that run alone (event-timed forward on one lane, "
+                                  "nothing else enqueued)")
+    if ms2 is not None:
+        roofline["side_by_side"] = {
+            "avg_launch_us": ms2[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],
+            "frac": gf / (ms2[pkg.K_GEMM] * 1e-3) / peak,
+            "note": "the same launches while another lane's forward shares the device: each "
+                    "lasts longer, two are in progress"}
     # the same launch against the HBM roof: at this batch the GEMM's flop-per-byte ratio is below
     # the machine's (peak flops / peak bytes), so HBM, not MFMA, is the roof above it
     alg_bytes = roofline["algorithmic_bytes_per_launch"]
