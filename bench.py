@@ -150,6 +150,40 @@ def search_workload(args, pkg, netgen):
     print(json.dumps(out))
 
 
+def netbench_workload(args, pkg, netgen):
+    """The reference's built-in benchmark of this path (Network::benchmark, GTP `netbench`,
+    reference src/Network.cpp:128-149): `threads` threads evaluate the empty board under
+    random symmetries, cache off, one blocking request each, `steps` x max batch evaluations.
+    Prints one JSON line of its own."""
+    B, F, blocks = args.batch, args.filters, args.blocks
+    prec = pkg.FP16 if args.precision == "fp16" else pkg.FP32
+    net = netgen.make_network(blocks, F, seed=2025)
+    w, h = netgen.prepare(net)
+    pipe = pkg.HIPScheduler(prec, B, device=0)
+    pipe.initialize(F)
+    pipe.push_weights(6, 18, F, w)
+    boards = np.full((1, 361), pkg.EMPTY, np.uint8)
+    pipe.netbench(h, boards, pkg.BLACK, args.threads, max(1, args.warmup) * B)
+    pipe.reset_stats()
+    done, secs = pipe.netbench(h, boards, pkg.BLACK, args.threads, args.steps * B)
+    st = pipe.stats()
+    pipe.close()
+    out = {
+        "metric": "netbench: evaluations/s through the request queue (Network::benchmark)",
+        "value": done / secs, "unit": "evals/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": secs / max(1, st["batches"]) * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 storage, f32 accumulate" if prec == pkg.FP16 else "f32",
+        "data": "synthetic (seeded random weights, the empty board under random symmetries)",
+        "config": {"workload": "%d threads, max batch %d, %dx%d %s, %d evaluations, heads on "
+                               "the calling threads" % (args.threads, B, blocks, F,
+                                                        args.precision, done)},
+        "batch_fill": st["requests"] / max(1, st["batch_slots"]), "batches": st["batches"],
+        "seconds": secs,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -165,8 +199,9 @@ def main():
     ap.add_argument("--lanes", type=int, default=0,
                     help="forward workload: batches kept on the device side by side; 0 = as "
                          "many as the handle has (2, or 3 up to batch 32)")
-    ap.add_argument("--workload", choices=["forward", "search"], default="forward",
-                    help="forward: the headline metric; search: BASELINE configs[4]")
+    ap.add_argument("--workload", choices=["forward", "search", "netbench"], default="forward",
+                    help="forward: the headline metric; search: BASELINE configs[4]; netbench: "
+                         "the reference's Network::benchmark (threads x single-position requests)")
     ap.add_argument("--threads", type=int, default=16, help="search threads (search workload)")
     ap.add_argument("--visits", type=int, default=1600)
     ap.add_argument("--moves", type=int, default=20)
@@ -199,9 +234,12 @@ def main():
                           "bytes_written": n * 4, "launches": 3}))
         return
     if args.batch is None:
-        args.batch = 64 if args.workload == "forward" else 32
+        args.batch = 32 if args.workload == "search" else 64
     if args.workload == "search":
         search_workload(args, pkg, netgen)
+        return
+    if args.workload == "netbench":
+        netbench_workload(args, pkg, netgen)
         return
 
     B, F, blocks = args.batch, args.filters, args.blocks

@@ -104,6 +104,17 @@ int lzhip_get_output_average(lzhip_handle* h, const lzhip_head_weights* heads,
                              const uint8_t* boards, int n_boards, int to_move,
                              float softmax_temp, float* policy, float* winrate);
 
+/* Network::benchmark (reference src/Network.cpp:128-149; the GTP command
+ * `netbench`, src/GTP.cpp:1055-1069): `threads` threads evaluate the given
+ * position, each time under a random symmetry and without the cache, until
+ * `iterations` evaluations have been started; every evaluation is one request
+ * through the scheduler with the heads on the calling thread, as in
+ * lzhip_get_output.  *evaluations is the number done (up to threads - 1 more than
+ * asked for, as in the reference), *seconds the wall time they took. */
+int lzhip_netbench(lzhip_handle* h, const lzhip_head_weights* heads, const uint8_t* boards,
+                   int n_boards, int to_move, int threads, int iterations, uint64_t seed,
+                   int* evaluations, double* seconds);
+
 int lzhip_search_default_config(lzhip_search_config* cfg);
 
 /* Self-play from the empty board with cfg->threads search threads calling the

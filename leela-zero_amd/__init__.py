@@ -45,7 +45,7 @@ EXPORTS = [
 # Every symbol include/lzhip_search.h declares.
 SEARCH_EXPORTS = [
     "lzhip_symmetry_index", "lzhip_gather_features", "lzhip_get_output",
-    "lzhip_get_output_average",
+    "lzhip_get_output_average", "lzhip_netbench",
     "lzhip_search_default_config", "lzhip_selfplay", "lzhip_board_replay",
 ]
 
@@ -161,6 +161,10 @@ def lib():
                                        _fp, _fp]
         L.lzhip_get_output_average.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights), _u8p,
                                                ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
+        L.lzhip_netbench.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights), _u8p,
+                                     ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                     ctypes.c_uint64, ctypes.POINTER(ctypes.c_int),
+                                     ctypes.POINTER(ctypes.c_double)]
         L.lzhip_search_default_config.argtypes = [ctypes.POINTER(SearchConfig)]
         L.lzhip_selfplay.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights),
                                      ctypes.POINTER(SearchConfig), ctypes.POINTER(SearchResult),
@@ -457,6 +461,21 @@ class HIPScheduler:
                                       ctypes.byref(win)))
         del keep
         return policy, win.value
+
+    def netbench(self, heads, boards, to_move, threads, iterations, seed=1):
+        """Network::benchmark (reference src/Network.cpp:128-149, GTP `netbench`): `threads`
+        threads evaluate the position under random symmetries, cache off, until
+        `iterations` evaluations have been started.  Returns (evaluations, seconds)."""
+        self._need()
+        c, keep = _c_heads(heads)
+        b, bp = _boards(boards)
+        done = ctypes.c_int()
+        secs = ctypes.c_double()
+        _check(lib().lzhip_netbench(self._h, c, bp, b.shape[0], int(to_move), int(threads),
+                                    int(iterations), int(seed), ctypes.byref(done),
+                                    ctypes.byref(secs)))
+        del keep
+        return done.value, secs.value
 
     def get_output_average(self, heads, boards, to_move, temperature=1.0):
         """Network::get_output with Ensemble::AVERAGE (reference

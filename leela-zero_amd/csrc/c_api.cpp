@@ -2,12 +2,16 @@
 // C++ exceptions into return codes; the message of the last failure is kept
 // per calling thread.
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <cmath>
 #include <cstring>
 #include <memory>
 #include <mutex>
 #include <stdexcept>
 #include <string>
+#include <thread>
+#include <vector>
 
 #include "forward_pipe.h"
 #include "hip_pipe.h"
@@ -330,6 +334,56 @@ int lzhip_get_output(lzhip_handle* h, const lzhip_head_weights* heads, const uin
     heads_on_host(*hw, pol.data(), val.data(), softmax_temp, p, winrate);
     for (int i = 0; i < go::kPoints; i++) policy[symmetry_index(symmetry, i)] = p[i];
     policy[go::kPoints] = p[go::kPoints];
+    return LZHIP_OK;
+    GUARD_END
+}
+
+int lzhip_netbench(lzhip_handle* h, const lzhip_head_weights* heads, const uint8_t* boards,
+                   int n_boards, int to_move, int threads, int iterations, uint64_t seed,
+                   int* evaluations, double* seconds) {
+    if (!h || !boards || !evaluations || !seconds) return fail(LZHIP_EINVAL, "null argument");
+    if (threads < 1 || threads > 4096 || iterations < 1)
+        return fail(LZHIP_EINVAL, "threads and iterations must be positive");
+    GUARD_BEGIN
+    const auto hw = resolve_heads(h, heads);
+    {   // the arguments are checked once, here, not in every thread
+        std::vector<float> probe(LZHIP_INPUT_SIZE);
+        const int rc = lzhip_gather_features(boards, n_boards, to_move, 0, probe.data());
+        if (rc != LZHIP_OK) return rc;
+    }
+    std::atomic<int> runcount{0}, halted{0};
+    std::mutex err_mu;
+    std::string err;
+    const auto t0 = std::chrono::steady_clock::now();
+    std::vector<std::thread> pool;
+    for (int t = 0; t < threads; t++)
+        pool.emplace_back([&, t] {
+            std::vector<float> in(LZHIP_INPUT_SIZE), pol(LZHIP_POL_SIZE), val(LZHIP_VAL_SIZE);
+            uint64_t st = seed + 0x9E3779B97F4A7C15ull * (uint64_t)(t + 1);
+            float p[go::kPoints + 1], win;
+            try {
+                while (runcount.load() < iterations && halted.load() == 0) {
+                    runcount++;
+                    st = st * 6364136223846793005ull + 1442695040888963407ull;
+                    const int sym = (int)(st >> 61);
+                    lzhip_gather_features(boards, n_boards, to_move, sym, in.data());
+                    if (h->sched->forward_raw(in.data(), pol.data(), val.data()) == LZHIP_EHALT) {
+                        halted++;
+                        break;
+                    }
+                    heads_on_host(*hw, pol.data(), val.data(), 1.0f, p, &win);
+                }
+            } catch (const std::exception& e) {
+                std::lock_guard<std::mutex> lk(err_mu);
+                err = e.what();
+                halted++;
+            }
+        });
+    for (auto& th : pool) th.join();
+    *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    *evaluations = runcount.load();
+    if (!err.empty()) throw std::runtime_error(err);
+    if (halted.load()) return fail(LZHIP_EHALT, "halted by drain");
     return LZHIP_OK;
     GUARD_END
 }

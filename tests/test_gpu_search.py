@@ -194,3 +194,36 @@ def test_selfplay_argument_checks(pkg, netgen, orc):
     with pytest.raises(ValueError):
         pipe.get_output(h, np.full((1, 361), 2, np.uint8), 0, symmetry=9)
     pipe.close()
+
+
+def test_netbench_counts_and_batches(pkg, netgen, orc):
+    """The reference's own benchmark of this path (Network::benchmark, GTP `netbench`): the
+    evaluations counted are those the scheduler answered, they come out of batches of
+    several callers, the count overshoots the request by fewer than the thread count, and
+    bad arguments and a drained pipe are reported."""
+    print("case: netbench", flush=True)
+    pipe, h, ref, h_ref = make(pkg, netgen, orc, 2, 64, 13, 1, 8)
+    b, boards = random_position(9, 30)
+    boards = np.array(boards, np.uint8)
+    pipe.reset_stats()
+    done, secs = pipe.netbench(h, boards, b.to_move, threads=12, iterations=300)
+    st = pipe.stats()
+    assert 300 <= done < 300 + 12 and secs > 0
+    assert st["requests"] == done
+    assert st["batches"] < done / 3            # 12 callers on a batch of 8: well-filled batches
+    assert st["max_batch_seen"] == 8
+    done1, _ = pipe.netbench(h, boards, b.to_move, threads=1, iterations=5)
+    assert done1 == 5
+    for bad in (dict(threads=0, iterations=5), dict(threads=2, iterations=0)):
+        with pytest.raises(ValueError):
+            pipe.netbench(h, boards, b.to_move, **bad)
+    with pytest.raises(ValueError):
+        pipe.netbench(h, boards, 2, threads=2, iterations=4)      # no such colour
+    pipe.drain()
+    with pytest.raises(pkg.NetworkHaltException):
+        pipe.netbench(h, boards, b.to_move, threads=3, iterations=10)
+    pipe.resume()
+    done2, _ = pipe.netbench(h, boards, b.to_move, threads=3, iterations=10)
+    assert 10 <= done2 < 13
+    pipe.close()
+
