@@ -104,6 +104,14 @@ int lzhip_get_output_average(lzhip_handle* h, const lzhip_head_weights* heads,
                              const uint8_t* boards, int n_boards, int to_move,
                              float softmax_temp, float* policy, float* winrate);
 
+/* Network::m_value_head_not_stm (reference src/Network.cpp:395-400): networks of
+ * weights-file format 2 give the value for black instead of for the side to
+ * move, and Network::get_output turns it round when white is to move
+ * (src/Network.cpp:797-802).  With `on` non-zero lzhip_get_output,
+ * lzhip_get_output_average and the search driver do the same; off by default.
+ * Set it before evaluations start. */
+int lzhip_set_value_head_not_stm(lzhip_handle* h, int on);
+
 /* Network::benchmark (reference src/Network.cpp:128-149; the GTP command
  * `netbench`, src/GTP.cpp:1055-1069): `threads` threads evaluate the given
  * position, each time under a random symmetry and without the cache, until

@@ -45,7 +45,7 @@ EXPORTS = [
 # Every symbol include/lzhip_search.h declares.
 SEARCH_EXPORTS = [
     "lzhip_symmetry_index", "lzhip_gather_features", "lzhip_get_output",
-    "lzhip_get_output_average", "lzhip_netbench",
+    "lzhip_get_output_average", "lzhip_netbench", "lzhip_set_value_head_not_stm",
     "lzhip_search_default_config", "lzhip_selfplay", "lzhip_board_replay",
 ]
 
@@ -161,6 +161,7 @@ def lib():
                                        _fp, _fp]
         L.lzhip_get_output_average.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights), _u8p,
                                                ctypes.c_int, ctypes.c_int, ctypes.c_float, _fp, _fp]
+        L.lzhip_set_value_head_not_stm.argtypes = [ctypes.c_void_p, ctypes.c_int]
         L.lzhip_netbench.argtypes = [ctypes.c_void_p, ctypes.POINTER(CHeadWeights), _u8p,
                                      ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                      ctypes.c_uint64, ctypes.POINTER(ctypes.c_int),
@@ -461,6 +462,13 @@ class HIPScheduler:
                                       ctypes.byref(win)))
         del keep
         return policy, win.value
+
+    def set_value_head_not_stm(self, on):
+        """Network::m_value_head_not_stm (weights-file format 2, reference
+        src/Network.cpp:395-400, :797-802): the value head speaks for black; get_output,
+        get_output_average and the search turn it round when white is to move."""
+        self._need()
+        _check(lib().lzhip_set_value_head_not_stm(self._h, 1 if on else 0))
 
     def netbench(self, heads, boards, to_move, threads, iterations, seed=1):
         """Network::benchmark (reference src/Network.cpp:128-149, GTP `netbench`): `threads`

@@ -28,6 +28,8 @@ struct lzhip_handle {
     // that run the heads on the calling thread with `heads == NULL`
     std::shared_ptr<const HeadWeights> host_heads;
     std::mutex heads_mu;
+    // Network::m_value_head_not_stm: set by the caller that read a format-2 weights file
+    std::atomic<bool> value_not_stm{false};
 };
 
 static thread_local std::string g_err;
@@ -334,6 +336,7 @@ int lzhip_get_output(lzhip_handle* h, const lzhip_head_weights* heads, const uin
     heads_on_host(*hw, pol.data(), val.data(), softmax_temp, p, winrate);
     for (int i = 0; i < go::kPoints; i++) policy[symmetry_index(symmetry, i)] = p[i];
     policy[go::kPoints] = p[go::kPoints];
+    if (h->value_not_stm.load() && to_move == go::WHITE) *winrate = 1.0f - *winrate;
     return LZHIP_OK;
     GUARD_END
 }
@@ -420,9 +423,15 @@ int lzhip_get_output_average(lzhip_handle* h, const lzhip_head_weights* heads,
         policy[go::kPoints] += p[go::kPoints] / (float)S;
         win += w / (float)S;
     }
-    *winrate = win;
+    *winrate = (h->value_not_stm.load() && to_move == go::WHITE) ? 1.0f - win : win;
     return LZHIP_OK;
     GUARD_END
+}
+
+int lzhip_set_value_head_not_stm(lzhip_handle* h, int on) {
+    if (!h) return fail(LZHIP_EINVAL, "null handle");
+    h->value_not_stm.store(on != 0);
+    return LZHIP_OK;
 }
 
 int lzhip_search_default_config(lzhip_search_config* cfg) {
@@ -455,7 +464,7 @@ int lzhip_selfplay(lzhip_handle* h, const lzhip_head_weights* heads,
         return fail(LZHIP_EINVAL, "threads in 1..4096, visits >= 1, moves >= 0, softmax_temp > 0");
     GUARD_BEGIN
     selfplay(*h->sched, resolve_heads(h, heads), *cfg, *result, moves_out,
-             moves_out ? moves_cap : 0);
+             moves_out ? moves_cap : 0, h->value_not_stm.load());
     return LZHIP_OK;
     GUARD_END
 }

@@ -241,6 +241,7 @@ Netresult NetworkFacade::get_output(const go::Position& pos, int symmetry, uint6
     }
     if (symmetry < 0) symmetry = (int)(next_rand(rng_state) >> 61);
     r = get_output_internal(pos, symmetry);
+    if (m_value_not_stm && pos.to_move() == go::WHITE) r.winrate = 1.0f - r.winrate;
     if (use_cache) m_cache.insert(key, r);
     return r;
 }
@@ -636,7 +637,8 @@ void UCTSearch::advance(int move) {
 // ---------------------------------------------------------------------------
 
 void selfplay(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads,
-              const lzhip_search_config& cfg, lzhip_search_result& out, int* moves, int moves_cap) {
+              const lzhip_search_config& cfg, lzhip_search_result& out, int* moves, int moves_cap,
+              bool value_head_not_stm) {
     std::memset(&out, 0, sizeof(out));
     auto* sched = dynamic_cast<HIPScheduler*>(&pipe);
     lzhip_stats before{};
@@ -645,6 +647,7 @@ void selfplay(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads,
     NetworkFacade net(pipe, std::move(heads), (size_t)std::max(cfg.cache_size, 0), cfg.softmax_temp);
     net.set_symmetry_probe(cfg.random_moves == 0);  // as the reference: not in randomised self-play
     net.set_device_heads(cfg.device_heads != 0);
+    net.set_value_head_not_stm(value_head_not_stm);
     UCTSearch search(net, cfg);
     go::Position pos;
     const auto t0 = std::chrono::steady_clock::now();

@@ -109,6 +109,10 @@ public:
     // executor has them); the calling thread then only gathers planes and
     // rotates the policy back.
     void set_device_heads(bool on);
+    // Networks of file format 2 give the value for black, not for the side to move
+    // (reference src/Network.cpp:395-400, :797-802): get_output then turns it round
+    // when white is to move.
+    void set_value_head_not_stm(bool on) { m_value_not_stm = on; }
     void drain() { m_pipe.drain(); }
     void resume() { m_pipe.resume(); }
     EvalCache& cache() { return m_cache; }
@@ -124,6 +128,7 @@ private:
     EvalCache m_cache;
     float m_temp;
     bool m_symmetry_probe = true;
+    bool m_value_not_stm = false;
     HIPScheduler* m_sched_heads = nullptr;   // set when the backend computes the heads
     std::atomic<uint64_t> m_evals{0}, m_probes{0}, m_probe_hits{0};
 };
@@ -199,7 +204,8 @@ private:
 // Plays cfg.moves moves of self-play from the empty board; fills `out` and, if
 // given, the move list.
 void selfplay(ForwardPipe& pipe, std::shared_ptr<const HeadWeights> heads,
-              const lzhip_search_config& cfg, lzhip_search_result& out, int* moves, int moves_cap);
+              const lzhip_search_config& cfg, lzhip_search_result& out, int* moves, int moves_cap,
+              bool value_head_not_stm = false);
 inline void selfplay(ForwardPipe& pipe, const lzhip_head_weights& heads,
                      const lzhip_search_config& cfg, lzhip_search_result& out, int* moves,
                      int moves_cap) {

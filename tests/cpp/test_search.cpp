@@ -180,6 +180,28 @@ static void test_unrotation() {
     }
 }
 
+// Format-2 networks give the value for black: get_output turns it round for white, also in
+// what it puts into the cache (reference src/Network.cpp:797-807).
+static void test_value_head_not_stm() {
+    HIPScheduler sched(std::make_unique<NeighbourNet>(4, 0));
+    Heads heads;
+    NetworkFacade plain(sched, heads.c, 0, 1.0f), flipped(sched, heads.c, 10, 1.0f);
+    flipped.set_value_head_not_stm(true);
+    go::Position pos;
+    uint64_t rng = 5;
+    const Netresult b0 = plain.get_output(pos, 0, rng, false);      // black to move
+    const Netresult b1 = flipped.get_output(pos, 0, rng, true);
+    CHECK(b0.winrate == b1.winrate);
+    pos.play(5 * 19 + 2);                                             // white to move
+    const Netresult w0 = plain.get_output(pos, 3, rng, false);
+    const Netresult w1 = flipped.get_output(pos, 3, rng, true);
+    CHECK(std::fabs(w1.winrate - (1.0f - w0.winrate)) < 1e-7f);
+    CHECK(std::fabs(w0.winrate - 0.5f) > 0.01f);                     // the flip is visible
+    for (int i = 0; i < kPoints; i++) CHECK(w0.policy[i] == w1.policy[i]);
+    const Netresult w2 = flipped.get_output(pos, 3, rng, true);      // from the cache
+    CHECK(flipped.cache_hits() == 1 && w2.winrate == w1.winrate);
+}
+
 static void test_symmetric_cache_probe() {
     HIPScheduler sched(std::make_unique<NeighbourNet>(4, 0));
     Heads heads;
@@ -398,6 +420,7 @@ static void test_selfplay_entry_and_failure() {
 int main() {
     std::printf("unrotation\n");
     test_unrotation();
+    test_value_head_not_stm();
     std::printf("symmetric cache probe\n");
     test_symmetric_cache_probe();
     std::printf("heads behind the pipe\n");

@@ -25,7 +25,7 @@ def test_library_exports_every_search_symbol(pkg):
     header = open(os.path.join(ROOT, "include", "lzhip_search.h")).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = sorted(set(re.findall(r"\b(lzhip_[a-z0-9_]+)\s*\(", header)))
-    assert len(declared) == 8
+    assert len(declared) == 9
     L = ctypes.CDLL(pkg.LIB_PATH)
     for name in declared:
         assert hasattr(L, name), name

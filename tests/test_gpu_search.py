@@ -227,3 +227,41 @@ def test_netbench_counts_and_batches(pkg, netgen, orc):
     assert 10 <= done2 < 13
     pipe.close()
 
+
+def test_value_head_of_format_2_networks(pkg, netgen, orc, tmp_path):
+    """A weights file of format 2 (value head speaks for black, reference
+    src/Network.cpp:395-400) round-trips through the file reader, and with the flag set
+    get_output, the average ensemble and the search turn the value round when white is to
+    move (src/Network.cpp:797-802) and leave the policy alone."""
+    print("case: value head not stm", flush=True)
+    net = netgen.make_network(1, 64, 17)
+    net.value_head_not_stm = True
+    path = str(tmp_path / "v2.txt.gz")
+    netgen.save_weights(net, path)
+    net2 = netgen.load_weights(path)
+    assert net2.value_head_not_stm
+    w, h = netgen.prepare(net2)
+    pipe = pkg.HIPScheduler(pkg.FP32, 8)
+    pipe.initialize(64)
+    pipe.push_weights(6, 18, 64, w)
+    b, boards = random_position(3, 31)            # 31 plies: white to move
+    assert b.to_move == pkg.WHITE
+    boards = np.array(boards, np.uint8)
+    p0, w0 = pipe.get_output(h, boards, b.to_move, 5)
+    a0, aw0 = pipe.get_output_average(h, boards, b.to_move)
+    pb0, wb0 = pipe.get_output(h, boards[1:], pkg.BLACK, 5)
+    pipe.set_value_head_not_stm(net2.value_head_not_stm)
+    p1, w1 = pipe.get_output(h, boards, b.to_move, 5)
+    a1, aw1 = pipe.get_output_average(h, boards, b.to_move)
+    pb1, wb1 = pipe.get_output(h, boards[1:], pkg.BLACK, 5)
+    assert abs(w1 - (1.0 - w0)) < 1e-6 and abs(aw1 - (1.0 - aw0)) < 1e-6
+    assert abs(w0 - 0.5) > 1e-3                    # the turn is visible
+    assert np.array_equal(p0, p1) and np.array_equal(a0, a1)
+    assert wb1 == wb0 and np.array_equal(pb0, pb1)  # black to move: unchanged
+    cfg = pkg.SearchConfig.default(threads=4, visits=60, moves=4, seed=3)
+    res, moves = pipe.selfplay(h, cfg)
+    assert res.moves_played == 4
+    pipe.set_value_head_not_stm(False)
+    assert pipe.get_output(h, boards, b.to_move, 5)[1] == w0
+    pipe.close()
+
