@@ -12,7 +12,9 @@ import subprocess
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "liblzoracle.so")
+# LZ_ORACLE_LIB: another build of lz_oracle.c to load instead (the test that compares an
+# -ffast-math build, the reference's own compiler setting, with this IEEE one)
+LIB_PATH = os.environ.get("LZ_ORACLE_LIB") or os.path.join(HERE, "liblzoracle.so")
 _fp = ctypes.POINTER(ctypes.c_float)
 _lib = None
 

@@ -212,3 +212,49 @@ def test_golden_fixtures(orc, netgen):
             hd = orc.heads(h, pol, val)
             assert max_abs(hd["policy"], g[tag + "_policy"][i]) < 1e-5
             assert abs(hd["value"] - g[tag + "_value"][i]) < 1e-5
+
+
+def test_fast_math_build_agrees(orc, netgen, tmp_path):
+    """The reference is compiled with -ffast-math (CMakeLists.txt:73, src/Makefile:6), the
+    oracle without.  The same source built both ways must agree far inside the 1e-4 parity
+    budget on a network whose heads are not saturated (6 blocks x 128 filters)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    fast = str(tmp_path / "liblzoracle_fast.so")
+    subprocess.run(["gcc", "-O3", "-mavx2", "-mfma", "-ffast-math", "-fPIC", "-std=c11",
+                    "-D_GNU_SOURCE", "-shared", "-o", fast,
+                    os.path.join(root, "oracle", "lz_oracle.c"), "-lm", "-lpthread", "-ldl"],
+                   check=True)
+    script = """
+import sys, numpy as np
+sys.path.insert(0, %r)
+import __graft_entry__ as entry
+orc = entry.load_oracle()
+entry.load_package()
+import leela_zero_amd.netgen as netgen
+orc.use_builtin()
+net = netgen.make_network(6, 128, seed=31)
+x = netgen.synthetic_inputs(2, seed=32)
+w, h = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+pipe = orc.OraclePipe(); pipe.initialize(128); pipe.push_weights(6, 18, 128, w)
+out = []
+for i in range(2):
+    pol, val = pipe.forward(x[i])
+    hd = orc.heads(h, pol, val)
+    out.append(np.concatenate([hd["policy"], [hd["value"]], pol.ravel(), val.ravel()]))
+np.save(sys.argv[1], np.array(out))
+""" % root
+    res = {}
+    for name, libpath in (("ieee", ""), ("fast", fast)):
+        env = dict(os.environ, LZ_ORACLE_LIB=libpath)
+        dst = str(tmp_path / (name + ".npy"))
+        subprocess.run([sys.executable, "-c", script, dst], check=True, env=env)
+        res[name] = np.load(dst)
+    a, b = res["ieee"], res["fast"]
+    assert max_abs(a[:, :363], b[:, :363]) < 1e-5          # policy and value
+    assert rel_l2(a[:, 363:], b[:, 363:]) < 1e-5           # raw planes
+    assert float(a[:, :362].max()) < 0.999 and int((a[:, :362] > 1e-4).sum()) >= 6   # heads not one-hot
+    assert float(np.abs(a[:, 362]).max()) < 0.999                                 # nor is the value
+
