@@ -183,7 +183,9 @@ private:
     std::atomic<int> m_outstanding{0};  // callers currently inside forward()
     int m_max_wait_us = -1;   // < 0: automatic
     int m_population = 1;     // callers seen around recent batches
-    int m_inflight = 0;       // positions in batches being executed
+    int m_inflight = 0;       // positions in batches assembled and not yet answered
+    int m_lanes = 1;          // batches the executor runs side by side
+    int m_exec_busy = 0;      // batches inside the executor right now
     double m_exec_us = 0.0;   // smoothed execution time of a batch
     std::string* m_fail_msg = nullptr;
     // statistics

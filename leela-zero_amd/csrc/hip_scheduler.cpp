@@ -59,9 +59,12 @@ void HIPScheduler::start_worker() {
     std::lock_guard<std::mutex> lk(m_mutex);
     if (m_running) return;
     m_running = true;
-    // As many workers as the executor runs batches side by side: while one waits for the
-    // device and hands results back, the others assemble and submit the next batches.
-    const int n = std::max(1, std::min(3, m_exec->max_concurrency()));
+    // One worker per batch the executor runs side by side, and one more: handing 64 results
+    // back (a wake-up per caller) takes a few hundred microseconds, during which that
+    // worker's share of the device would sit idle; the spare worker has the next full
+    // batch assembled by then and submits it the moment the executor is free.
+    m_lanes = std::max(1, std::min(3, m_exec->max_concurrency()));
+    const int n = m_lanes + 1;
     for (int i = 0; i < n; i++) m_workers.emplace_back(&HIPScheduler::worker, this);
 }
 
@@ -237,6 +240,15 @@ void HIPScheduler::worker() {
             const int cap_us = m_max_wait_us >= 0
                                    ? m_max_wait_us
                                    : std::max(50, std::min(5000, (int)(m_exec_us * 0.5)));
+            // Every executor slot taken: only a full batch is worth assembling ahead of
+            // time; otherwise wait for a slot and decide then.
+            if (m_exec_busy >= m_lanes) {
+                m_cv.wait(lk, [&] {
+                    return !m_running || m_queue.empty() || m_exec_busy < m_lanes ||
+                           (int)m_queue.size() >= m_max_batch;
+                });
+                if (!m_running) return;
+            }
             // Callers known to exist: those seen around recent batches, or inside
             // forward() right now.  If they all fit one batch, a second batch next
             // to the one in flight would only split them into two small ones that
@@ -290,6 +302,12 @@ void HIPScheduler::worker() {
             for (int i = 0; i < n; i++)
                 std::memcpy(in.data() + (size_t)i * kInSize, batch[i]->in, sizeof(float) * kInSize);
         }
+        {
+            // the executor takes m_lanes batches at a time
+            std::unique_lock<std::mutex> lk(m_mutex);
+            m_cv.wait(lk, [&] { return m_exec_busy < m_lanes; });
+            m_exec_busy++;
+        }
         int outcome = 1;
         const auto t0 = std::chrono::steady_clock::now();
         try {
@@ -315,6 +333,7 @@ void HIPScheduler::worker() {
             // callers in flight plus those that queued up meanwhile; forgets slowly
             m_population = std::max(m_outstanding.load(), m_population - 1);
             m_inflight -= n;
+            m_exec_busy--;
         }
         m_cv.notify_all();  // a collector may be waiting for the device to come free
         m_batches++;
