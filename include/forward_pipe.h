@@ -73,8 +73,9 @@ class BatchExecutor {
 public:
     virtual ~BatchExecutor() = default;
     virtual int max_batch() const = 0;
-    // How many forward_batch calls may run at the same time (the scheduler
-    // starts that many worker threads, at most two).
+    // How many forward_batch calls may run at the same time.  The scheduler never
+    // has more than that many (at most three) inside the executor; it starts one
+    // worker thread more, which assembles the next batch meanwhile.
     virtual int max_concurrency() const { return 1; }
     // in [n][18*361] -> pol [n][722], val [n][361]; throws std::runtime_error.
     virtual void forward_batch(int n, const float* in, float* pol, float* val) = 0;
