@@ -127,13 +127,14 @@ def test_forward_parity(pkg, netgen, orc, blocks, filters, batch, precision):
 
 
 @pytest.mark.parametrize("precision", [0, 1])
-@pytest.mark.parametrize("batch", [64, 41, 24, 10, 2])
+@pytest.mark.parametrize("batch", [64, 52, 41, 33, 24, 10, 2])
 def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
-    """256 filters at batch sizes that select the different kernel shapes (GEMM: 256x256
-    tiles in two passes from 41 boards up, persistent 128x128 tiles below, 128x64 tiles
-    for the smallest batches; fused transform: 64, 32 or 16 channels per work-group), in
-    both precisions, including batches whose tile count is not a multiple of any tile
-    height."""
+    """256 filters at batch sizes on both sides of every change of kernel shape (GEMM, fp16:
+    256x256 tiles in two passes from 52 boards, persistent 128x128 tiles from 41, 128x64
+    tiles with permuted LDS rows below; fp32: 256x256 from 41, 128x128 from 21, 128x64 with
+    padded rows below; fused transform: 64 channels per work-group from 33 boards, 32 from 6,
+    16 below), in both precisions, including batches whose tile count is not a multiple of
+    any tile height."""
     print("case: wide 3x256 b%d precision=%d" % (batch, precision), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 256, 3000, precision, batch)
     x = netgen.synthetic_inputs(batch, seed=batch)
