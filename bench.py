@@ -104,7 +104,7 @@ def calibrate_heads(pipe, netgen, h, batch):
 
 
 def search_workload(args, pkg, netgen):
-    """BASELINE configs[4]: tree search with `threads` search threads driving the
+    """The search workload: tree search with `threads` search threads driving the
     scheduler at max batch `batch`; every move `visits` root visits, `moves` moves of
     self-play from the empty board.  Prints one JSON line of its own."""
     B, F, blocks = args.batch, args.filters, args.blocks
@@ -129,7 +129,7 @@ def search_workload(args, pkg, netgen):
     pipe.close()
     fill = res.sched.requests / max(1, res.sched.batch_slots)
     out = {
-        "metric": "search visits/sec and NN batch-fill ratio (BASELINE configs[4])",
+        "metric": "search visits/sec and NN batch-fill ratio",
         "value": res.visits_per_s, "unit": "visits/s", "n_gpus": 1, "steps": res.moves_played,
         "warmup": 1, "ms_per_step": res.seconds / max(1, res.moves_played) * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -200,7 +200,7 @@ def main():
                     help="forward workload: batches kept on the device side by side; 0 = as "
                          "many as the handle has (2, or 3 up to batch 32)")
     ap.add_argument("--workload", choices=["forward", "search", "netbench"], default="forward",
-                    help="forward: the headline metric; search: BASELINE configs[4]; netbench: "
+                    help="forward: the headline metric; search: visits/s of a multi-threaded tree search; netbench: "
                          "the reference's Network::benchmark (threads x single-position requests)")
     ap.add_argument("--threads", type=int, default=16, help="search threads (search workload)")
     ap.add_argument("--visits", type=int, default=1600)
@@ -396,7 +396,7 @@ def main():
         "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 storage, f32 accumulate" if prec == pkg.FP16 else "f32",
         "data": "synthetic",
-        "config": {"workload": "%d blocks x %d filters, %s, batch %d (BASELINE configs[3] when "
+        "config": {"workload": "%d blocks x %d filters, %s, batch %d (the headline configuration when "
                                "40x256 fp16 b64), %d conv layers + 1x1 heads per step"
                                % (blocks, F, args.precision, B, nl),
                    "inputs": "device-resident fp32 NCHW [%d][18][361]" % B,

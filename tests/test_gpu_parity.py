@@ -111,10 +111,10 @@ def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None):
 
 @pytest.mark.parametrize("blocks,filters,batch,precision", [
     (1, 8, 3, 0),       # the shape of the reference's test network (1 block x 8 filters)
-    (6, 128, 1, 0),     # config 0: 6x128 fp32 batch 1
-    (15, 192, 8, 0),    # config 1: 15x192 fp32 batch 8
+    (6, 128, 1, 0),     # the smallest benchmark configuration: 6x128 fp32 batch 1
+    (15, 192, 8, 0),    # 15x192 fp32 batch 8
     (1, 8, 3, 1),
-    (6, 128, 4, 1),     # config-0-sized net in fp16: the non-saturated fp16 check
+    (6, 128, 4, 1),     # the same small net in fp16: the non-saturated fp16 check
     (2, 96, 5, 1),
 ])
 def test_forward_parity(pkg, netgen, orc, blocks, filters, batch, precision):
@@ -144,7 +144,8 @@ def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
 
 @pytest.mark.parametrize("blocks,filters,batch", [(20, 256, 32), (40, 256, 64)])
 def test_forward_parity_deep_fp16(pkg, netgen, orc, blocks, filters, batch):
-    """Configs 2 and 3 at full size; the oracle checks three positions of the batch."""
+    """The two large fp16 benchmark configurations (20x256 batch 32, 40x256 batch 64) at full
+    size; the oracle checks three positions of the batch."""
     print("case: deep fp16 %dx%d b%d" % (blocks, filters, batch), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, blocks, filters, 2000 + blocks,
                                        pkg.FP16, batch)
