@@ -66,6 +66,21 @@ typedef struct lzhip_stats {
  * HIP runtime is unavailable: there is no CPU fallback. */
 int lzhip_create(int filters, int precision, int max_batch, int device, lzhip_handle** out);
 
+/* Network::initialize from a weights file (reference src/Network.cpp:351-405
+ * load_network_file, :225-349 load_v1_network, :540-576 preparation): reads a
+ * Leela Zero weights file (text, plain or gzip, format 1 or 2), detects filters and
+ * residual blocks from it as the engine does, applies the Winograd transform of the
+ * filters, 1/sqrt(var + 1e-5) and the folding of the conv biases into the batch-norm
+ * means, creates the handle and pushes tower weights and head parameters
+ * (lzhip_push_heads); format 2 sets lzhip_set_value_head_not_stm.  A file the
+ * engine would refuse gives LZHIP_EINVAL with the engine's message ("Weights file is
+ * the wrong version.", "Inconsistent number of weights in the file.", "Failed to
+ * parse weight file. Error on line N.", "The weights file is not for 19x19 boards.",
+ * "Could not open weights file: ...") before any device is touched.  filters and
+ * blocks may be NULL. */
+int lzhip_create_from_file(const char* path, int precision, int max_batch, int device,
+                           lzhip_handle** out, int* filters, int* blocks);
+
 /* Destructor of the backend (reference src/OpenCLScheduler.cpp:134-144):
  * wakes and joins the worker, pending requests finish with LZHIP_EHALT. */
 int lzhip_destroy(lzhip_handle* h);

@@ -34,7 +34,7 @@ KERNEL_CLASSES = ["pack_input", "in_transform", "gemm", "out_transform", "head_c
 
 # Every symbol include/lzhip.h declares.
 EXPORTS = [
-    "lzhip_create", "lzhip_destroy", "lzhip_push_weights", "lzhip_forward",
+    "lzhip_create", "lzhip_create_from_file", "lzhip_destroy", "lzhip_push_weights", "lzhip_forward",
     "lzhip_forward_batch", "lzhip_forward_batch_device", "lzhip_lanes",
     "lzhip_forward_batch_device_lane", "lzhip_sync", "lzhip_stream",
     "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats", "lzhip_push_heads",
@@ -132,6 +132,10 @@ def lib():
         L.lzhip_stream.restype = ctypes.c_void_p
         L.lzhip_stream.argtypes = [ctypes.c_void_p]
         L.lzhip_create.argtypes = [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_void_p)]
+        L.lzhip_create_from_file.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int,
+                                             ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
+                                             ctypes.POINTER(ctypes.c_int),
+                                             ctypes.POINTER(ctypes.c_int)]
         L.lzhip_destroy.argtypes = [ctypes.c_void_p]
         L.lzhip_push_weights.argtypes = [ctypes.c_void_p, ctypes.c_int, _fpp, _fpp, _fpp, _fp, _fp]
         L.lzhip_forward.argtypes = [ctypes.c_void_p, _fp, _fp, _fp]
@@ -297,6 +301,22 @@ class HIPScheduler:
         self.n_layers = 0
         self.filters = 0
         self._keep = None
+
+    @classmethod
+    def from_file(cls, path, precision=FP16, max_batch=1, device=0):
+        """Network::initialize from a weights file (reference src/Network.cpp:225-405,
+        :540-576): plain or gzip text, format 1 or 2; tower and head parameters are
+        pushed, so `heads=None` works in the callers above forward()."""
+        self = cls(precision, max_batch, device)
+        h = ctypes.c_void_p()
+        f, b = ctypes.c_int(), ctypes.c_int()
+        _check(lib().lzhip_create_from_file(os.fsencode(path), self.precision, self.max_batch,
+                                            self.device, ctypes.byref(h), ctypes.byref(f),
+                                            ctypes.byref(b)))
+        self._h = h
+        self.filters = f.value
+        self.n_layers = 1 + 2 * b.value
+        return self
 
     # -- ForwardPipe interface -------------------------------------------
     def initialize(self, channels):

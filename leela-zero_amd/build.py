@@ -14,6 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "liblzhip.so")
 
 SOURCES = ["kernels.hip", "hip_pipe.hip", "hip_scheduler.cpp", "goboard.cpp", "search.cpp",
+           "weights_file.cpp",
            "c_api.cpp"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are kept out of the generated code.
@@ -47,7 +48,7 @@ def build(verbose=False):
         if verbose and err.strip():
             print(err, file=sys.stderr)
         objs.append(obj)
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-lpthread"]
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-lpthread", "-lz"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)

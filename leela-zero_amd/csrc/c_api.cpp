@@ -18,6 +18,7 @@
 #include "lzhip.h"
 #include "lzhip_search.h"
 #include "search.h"
+#include "weights_file.h"
 
 using namespace lzhip;
 
@@ -73,6 +74,43 @@ int lzhip_create(int filters, int precision, int max_batch, int device, lzhip_ha
     h->sched = std::make_unique<HIPScheduler>(std::unique_ptr<BatchExecutor>(pipe.release()));
     h->pipe = raw;
     *out = h.release();
+    return LZHIP_OK;
+    GUARD_END
+}
+
+int lzhip_create_from_file(const char* path, int precision, int max_batch, int device,
+                           lzhip_handle** out, int* filters, int* blocks) {
+    if (!path || !out) return fail(LZHIP_EINVAL, "null argument");
+    *out = nullptr;
+    GUARD_BEGIN
+    const WeightsFile wf = load_weights_file(path);   // before any device is touched
+    if (filters) *filters = wf.filters;
+    if (blocks) *blocks = wf.blocks;
+    lzhip_handle* h = nullptr;
+    int rc = lzhip_create(wf.filters, precision, max_batch, device, &h);
+    if (rc != LZHIP_OK) return rc;
+    const size_t nl = wf.U.size();
+    std::vector<const float*> U(nl), mean(nl), scale(nl);
+    for (size_t l = 0; l < nl; l++) {
+        U[l] = wf.U[l].data();
+        mean[l] = wf.bn_mean[l].data();
+        scale[l] = wf.bn_scale[l].data();
+    }
+    rc = lzhip_push_weights(h, (int)nl, U.data(), mean.data(), scale.data(), wf.conv_pol_w.data(),
+                            wf.conv_val_w.data());
+    if (rc == LZHIP_OK)
+        rc = lzhip_push_heads(h, wf.bn_pol_mean.data(), wf.bn_pol_scale.data(), wf.ip_pol_w.data(),
+                              wf.ip_pol_b.data(), wf.bn_val_mean.data(), wf.bn_val_scale.data(),
+                              wf.ip1_val_w.data(), wf.ip1_val_b.data(), wf.ip2_val_w.data(),
+                              wf.ip2_val_b.data());
+    if (rc != LZHIP_OK) {
+        const std::string keep = g_err;
+        lzhip_destroy(h);
+        g_err = keep;
+        return rc;
+    }
+    h->value_not_stm.store(wf.value_head_not_stm);
+    *out = h;
     return LZHIP_OK;
     GUARD_END
 }

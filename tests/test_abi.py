@@ -123,3 +123,56 @@ def test_reference_weights_fixture_loads(netgen, orc, tmp_path):
     hd = orc.heads(h, pol, val)
     assert abs(float(hd["policy"].sum()) - 1.0) < 1e-5 and 0.0 < hd["winrate"] < 1.0
     assert hd["policy"].max() < 0.9      # a real network: not a saturated one-hot
+
+
+def test_create_from_file_refuses_what_the_engine_refuses(pkg, netgen, tmp_path):
+    """lzhip_create_from_file reads the file before it touches a device, so the refusals of
+    the engine's reader (reference src/Network.cpp:225-405) can be checked here: missing file,
+    wrong version, a line count that is not 19 + 8 blocks, a token that is no number, a policy
+    layer of another board size.  A good file gets as far as the device (which this host
+    lacks, or which then serves it)."""
+    import gzip
+    import torch
+    good = os.path.join(ROOT, "tests", "golden", "0k.txt.gz")
+    lines = gzip.open(good, "rt").read().splitlines()
+    assert len(lines) == 1 + 4 + 14 + 8 * 1
+
+    def attempt(path):
+        return pkg.HIPScheduler.from_file(str(path), pkg.FP32, 2)
+
+    def write(name, ls):
+        path = tmp_path / name
+        path.write_text("\n".join(ls) + "\n")
+        return path
+
+    with pytest.raises(ValueError, match="Could not open weights file"):
+        attempt(tmp_path / "missing.txt")
+    with pytest.raises(ValueError, match="wrong version"):
+        attempt(write("v3.txt", ["3"] + lines[1:]))
+    with pytest.raises(ValueError, match="wrong version"):
+        attempt(write("empty.txt", [""]))
+    with pytest.raises(ValueError, match="Inconsistent number of weights"):
+        attempt(write("short.txt", lines[:-1]))
+    bad = list(lines)
+    bad[7] = bad[7].replace(" ", " x ", 1)
+    with pytest.raises(ValueError, match="Error on line 8"):
+        attempt(write("token.txt", bad))
+    other = list(lines)
+    other[1 + 4 + 8 + 4] = " ".join(other[1 + 4 + 8 + 4].split()[:-362])   # one move fewer
+    with pytest.raises(ValueError, match="not for 19x19 boards"):
+        attempt(write("board.txt", other))
+    narrow = list(lines)
+    narrow[3] = " ".join(narrow[3].split()[:-1])                          # a mean goes missing
+    with pytest.raises(ValueError, match="Inconsistent number of weights"):
+        attempt(write("narrow.txt", narrow))
+    # plain text and gzip are both read; without a device the good file ends at the device
+    plain = write("plain.txt", lines)
+    for path in (good, plain):
+        if torch.cuda.is_available():
+            pipe = attempt(path)
+            assert (pipe.filters, pipe.n_layers) == (8, 3)
+            pipe.close()
+        else:
+            with pytest.raises(pkg.LzhipError):
+                attempt(path)
+

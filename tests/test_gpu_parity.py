@@ -198,6 +198,45 @@ def test_reference_weights_file_on_device(pkg, netgen, orc, precision):
     pipe.close()
 
 
+def test_handle_created_from_a_weights_file(pkg, netgen, orc, tmp_path):
+    """lzhip_create_from_file (reading, Winograd transform, bias folding, push of tower and
+    heads in one call) gives bit for bit what the Python reader plus push_weights/push_heads
+    give, for the reference's own test file (gzip) and for a seeded 2-block net written as
+    format 2 in plain text; the heads it pushed serve `heads=None`, and format 2 turns the
+    value round for white."""
+    import os
+    print("case: create from file", flush=True)
+    x = netgen.synthetic_inputs(5, seed=41)
+    ref_file = os.path.join(os.path.dirname(__file__), "golden", "0k.txt.gz")
+    net2 = netgen.make_network(2, 24, 43)
+    net2.value_head_not_stm = True
+    v2_file = str(tmp_path / "v2.txt")
+    netgen.save_weights(net2, v2_file)
+    for path in (ref_file, v2_file):
+        net = netgen.load_weights(path)
+        w, h = netgen.prepare(net)
+        a = pkg.HIPScheduler(pkg.FP32, 8)
+        a.initialize(net.filters)
+        a.push_weights(6, 18, net.filters, w)
+        a.push_heads(h)
+        b = pkg.HIPScheduler.from_file(path, pkg.FP32, 8)
+        assert (b.filters, b.n_layers) == (net.filters, net.n_layers)
+        pa, pb = a.forward_batch(x), b.forward_batch(x)
+        assert np.array_equal(pa[0], pb[0]) and np.array_equal(pa[1], pb[1])
+        ea, eb = a.evaluate_batch(x), b.evaluate_batch(x)
+        assert np.array_equal(ea[0], eb[0]) and np.array_equal(ea[1], eb[1])
+        # callers above forward(): the heads pushed from the file, and the format-2 flag
+        boards = np.full((1, 361), pkg.EMPTY, np.uint8)
+        boards[0, 72] = pkg.BLACK
+        pol_a, win_a = a.get_output(h, boards, pkg.WHITE, 2)
+        pol_b, win_b = b.get_output(None, boards, pkg.WHITE, 2)
+        assert np.array_equal(pol_a, pol_b)
+        want = 1.0 - win_a if net.value_head_not_stm else win_a
+        assert abs(win_b - want) < 1e-7
+        a.close()
+        b.close()
+
+
 @pytest.mark.parametrize("precision", [0, 1])
 def test_batch_composition_does_not_change_results(pkg, netgen, orc, precision):
     """A position evaluated alone, in a partial batch and in a full batch gives
