@@ -157,11 +157,16 @@ def netbench_workload(args, pkg, netgen):
     Prints one JSON line of its own."""
     B, F, blocks = args.batch, args.filters, args.blocks
     prec = pkg.FP16 if args.precision == "fp16" else pkg.FP32
-    net = netgen.make_network(blocks, F, seed=2025)
-    w, h = netgen.prepare(net)
-    pipe = pkg.HIPScheduler(prec, B, device=0)
-    pipe.initialize(F)
-    pipe.push_weights(6, 18, F, w)
+    if args.weights:
+        # a network file, read and prepared by the library as the engine reads it
+        pipe = pkg.HIPScheduler.from_file(args.weights, prec, B, device=0)
+        h, F, blocks = None, pipe.filters, (pipe.n_layers - 1) // 2
+    else:
+        net = netgen.make_network(blocks, F, seed=2025)
+        w, h = netgen.prepare(net)
+        pipe = pkg.HIPScheduler(prec, B, device=0)
+        pipe.initialize(F)
+        pipe.push_weights(6, 18, F, w)
     boards = np.full((1, 361), pkg.EMPTY, np.uint8)
     pipe.netbench(h, boards, pkg.BLACK, args.threads, max(1, args.warmup) * B)
     pipe.reset_stats()
@@ -174,7 +179,8 @@ def netbench_workload(args, pkg, netgen):
         "warmup": args.warmup, "ms_per_step": secs / max(1, st["batches"]) * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 storage, f32 accumulate" if prec == pkg.FP16 else "f32",
-        "data": "synthetic (seeded random weights, the empty board under random symmetries)",
+        "data": ("weights file %s" % args.weights if args.weights else
+                 "synthetic (seeded random weights)") + ", the empty board under random symmetries",
         "config": {"workload": "%d threads, max batch %d, %dx%d %s, %d evaluations, heads on "
                                "the calling threads" % (args.threads, B, blocks, F,
                                                         args.precision, done)},
@@ -208,6 +214,9 @@ def main():
     ap.add_argument("--no-tree-reuse", action="store_true")
     ap.add_argument("--device-heads", action="store_true",
                     help="search workload: heads computed on the device, not on the search threads")
+    ap.add_argument("--weights", default=None, metavar="FILE",
+                    help="netbench workload: a Leela Zero weights file instead of the seeded "
+                         "random network")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy kernel of MIB mebibytes three times "
                          "(known traffic, for scaling the FETCH_SIZE / WRITE_SIZE counters)")
