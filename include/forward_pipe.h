@@ -146,6 +146,8 @@ public:
     int evaluate_raw(const float* in, float temperature, float* policy, float* value);
 
     BatchExecutor* executor() { return m_exec.get(); }
+    // Callers inside forward() right now (queued, in a batch, or about to return).
+    int outstanding() const { return m_outstanding.load(); }
     lzhip_stats stats();
     void reset_stats();
     // Upper bound, in microseconds, of the grace period the worker grants a

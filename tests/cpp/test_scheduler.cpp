@@ -16,8 +16,10 @@
 //     batch per round instead of two alternating partial ones.
 #include <atomic>
 #include <chrono>
+#include <condition_variable>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 #include <stdexcept>
 #include <thread>
 #include <vector>
@@ -60,6 +62,10 @@ public:
         } in_flight(this);
         if (n < 1 || n > m_mb) { oversize = true; }
         if (fail_next.exchange(false)) throw std::runtime_error("injected failure");
+        {   // a closed gate keeps every batch inside the executor until the test opens it
+            std::unique_lock<std::mutex> lk(m_gate_mu);
+            m_gate_cv.wait(lk, [&] { return m_gate_open; });
+        }
         std::this_thread::sleep_for(std::chrono::microseconds(m_delay));
         for (int b = 0; b < n; b++) {
             const float* x = in + (size_t)b * LZHIP_INPUT_SIZE;
@@ -69,10 +75,20 @@ public:
         calls++;
         positions += n;
     }
+    void set_gate(bool open) {
+        {
+            std::lock_guard<std::mutex> lk(m_gate_mu);
+            m_gate_open = open;
+        }
+        m_gate_cv.notify_all();
+    }
     std::atomic<bool> oversize{false}, fail_next{false};
     std::atomic<int> calls{0}, positions{0}, inside{0}, max_inside{0};
 private:
     int m_mb, m_delay, m_conc;
+    std::mutex m_gate_mu;
+    std::condition_variable m_gate_cv;
+    bool m_gate_open = true;
 };
 
 // Takes bit-packed planes; the answer depends on every input value:
@@ -210,21 +226,32 @@ static void test_population_batches(int concurrency) {
     CHECK(mean >= 9.0);
 }
 
+// drain() while batches sit inside the executor and requests wait in the queue.  The
+// executor is held on a gate, so "queued while a batch is inside" is a state the test
+// waits for, not a guess about timing: with `concurrency` batches inside and the spare
+// worker holding at most one assembled batch more, at most (concurrency + 1) * max_batch
+// of the 32 requests have left the queue when drain() runs; all others must halt.
 static void test_drain_resume(int concurrency) {
-    auto* fe = new FakeExec(4, 20000, concurrency);  // slow executor: requests pile up in the queue
+    const int mb = 4, callers = 32;
+    auto* fe = new FakeExec(mb, 100, concurrency);
     HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
     s.set_max_wait_us(0);
+    fe->set_gate(false);
     std::atomic<int> ok{0}, halted{0};
     std::vector<std::thread> th;
-    for (int t = 0; t < 16; t++) th.emplace_back([&, t] { one_call(s, (float)t, 1.0f, ok, halted); });
-    std::this_thread::sleep_for(std::chrono::milliseconds(5));
+    for (int t = 0; t < callers; t++)
+        th.emplace_back([&, t] { one_call(s, (float)t, 1.0f, ok, halted); });
+    while (s.outstanding() < callers || fe->inside < concurrency) std::this_thread::yield();
     s.drain();
-    for (auto& t : th) t.join();
-    CHECK(ok + halted == 16);
-    CHECK(halted >= 1);  // the slow executor cannot have served all 16 in 5 ms
-    // while drained every new call halts immediately
+    // a call made while drained halts at once, also with batches still inside the executor
     one_call(s, 1.0f, 2.0f, ok, halted);
-    CHECK(ok + halted == 17);
+    CHECK(ok == 0 && halted >= 1);
+    fe->set_gate(true);
+    for (auto& t : th) t.join();
+    CHECK(ok + halted == callers + 1);
+    CHECK(ok >= 1 && ok <= (concurrency + 1) * mb);
+    CHECK(halted >= callers + 1 - (concurrency + 1) * mb);
+    CHECK(fe->max_inside == concurrency);
     const int halted_before = halted;
     s.resume();
     one_call(s, 3.0f, 4.0f, ok, halted);
