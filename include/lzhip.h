@@ -131,6 +131,22 @@ int lzhip_forward_batch_device(lzhip_handle* h, int n, const void* d_in, void* d
 int lzhip_lanes(lzhip_handle* h);
 int lzhip_forward_batch_device_lane(lzhip_handle* h, int lane, int n, const void* d_in,
                                     void* d_pol, void* d_val);
+/* No counterpart in the reference.  For callers that cannot allocate device memory at
+ * the time of the call -- code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc: lzhip_forward_batch_device (lane 0's stream, same arguments,
+ * same results bit for bit) with every working buffer of the forward (packed planes,
+ * activations, the Winograd tile arrays V and M) in a static device array of
+ * 28 485 632 bytes that each GPU holds from library load to process end, instead of
+ * the lane's allocated buffers.  The call launches kernels and nothing else.
+ * Limits: 1 <= n <= LZHIP_NOALLOC_MAX_BATCH (and <= max_batch), networks of up to
+ * LZHIP_NOALLOC_MAX_FILTERS filters; anything larger returns LZHIP_EINVAL with a
+ * message.  All calls on one GPU share the array, from whatever handle: calls that
+ * overlap on that GPU race (calls on one handle are ordered by its stream).
+ * Returns without waiting; lzhip_sync waits. */
+#define LZHIP_NOALLOC_MAX_BATCH 8
+#define LZHIP_NOALLOC_MAX_FILTERS 256
+int lzhip_forward_batch_device_noalloc(lzhip_handle* h, int n, const void* d_in, void* d_pol,
+                                       void* d_val);
 /* Waits for the work enqueued on every lane. */
 int lzhip_sync(lzhip_handle* h);
 /* The hipStream_t of lane 0 (for callers that record events). */

@@ -36,7 +36,7 @@ KERNEL_CLASSES = ["pack_input", "in_transform", "gemm", "out_transform", "head_c
 EXPORTS = [
     "lzhip_create", "lzhip_create_from_file", "lzhip_destroy", "lzhip_push_weights", "lzhip_forward",
     "lzhip_forward_batch", "lzhip_forward_batch_device", "lzhip_lanes",
-    "lzhip_forward_batch_device_lane", "lzhip_sync", "lzhip_stream",
+    "lzhip_forward_batch_device_lane", "lzhip_forward_batch_device_noalloc", "lzhip_sync", "lzhip_stream",
     "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats", "lzhip_push_heads",
     "lzhip_evaluate_batch", "lzhip_forward_eval", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
     "lzhip_debug_layer", "lzhip_get_act_scales", "lzhip_profile_forward", "lzhip_last_error",
@@ -141,6 +141,8 @@ def lib():
         L.lzhip_forward.argtypes = [ctypes.c_void_p, _fp, _fp, _fp]
         L.lzhip_forward_batch.argtypes = [ctypes.c_void_p, ctypes.c_int, _fp, _fp, _fp]
         L.lzhip_forward_batch_device.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 3
+        L.lzhip_forward_batch_device_noalloc.argtypes = ([ctypes.c_void_p, ctypes.c_int]
+                                                        + [ctypes.c_void_p] * 3)
         L.lzhip_lanes.argtypes = [ctypes.c_void_p]
         L.lzhip_forward_batch_device_lane.argtypes = ([ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
                                                       + [ctypes.c_void_p] * 3)
@@ -394,6 +396,12 @@ class HIPScheduler:
         self._need()
         _check(lib().lzhip_forward_batch_device_lane(self._h, int(lane), int(n), d_in, d_pol,
                                                      d_val))
+
+    def forward_batch_device_noalloc(self, n, d_in, d_pol, d_val):
+        """forward_batch_device on lane 0 with the working buffers in the library's static
+        device array: no allocation on the way.  n <= 8, up to 256 filters."""
+        self._need()
+        _check(lib().lzhip_forward_batch_device_noalloc(self._h, int(n), d_in, d_pol, d_val))
 
     def sync(self):
         self._need()

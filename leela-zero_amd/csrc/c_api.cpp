@@ -173,6 +173,16 @@ int lzhip_forward_batch_device_lane(lzhip_handle* h, int lane, int n, const void
     GUARD_END
 }
 
+int lzhip_forward_batch_device_noalloc(lzhip_handle* h, int n, const void* d_in, void* d_pol,
+                                       void* d_val) {
+    if (!h || !d_in || !d_pol || !d_val) return fail(LZHIP_EINVAL, "null argument");
+    GUARD_BEGIN
+    h->pipe->forward_device_static(n, static_cast<const float*>(d_in),
+                                   static_cast<float*>(d_pol), static_cast<float*>(d_val));
+    return LZHIP_OK;
+    GUARD_END
+}
+
 int lzhip_sync(lzhip_handle* h) {
     if (!h) return fail(LZHIP_EINVAL, "null handle");
     GUARD_BEGIN

@@ -29,6 +29,10 @@ public:
     virtual int lanes() const = 0;
     virtual void forward_device(int lane, int n, const float* d_in, float* d_pol,
                                 float* d_val) = 0;
+    // forward_device on lane 0's stream with the working buffers in a static device array
+    // (no allocation anywhere on the way); small batches and nets only, see lzhip.h.
+    virtual void forward_device_static(int n, const float* d_in, float* d_pol,
+                                       float* d_val) = 0;
     virtual void sync() = 0;
     virtual void* stream() = 0;
 

@@ -31,6 +31,46 @@ typedef _Float16 half_t;
 
 static inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+// Working memory of the entry point that allocates nothing (forward_device_static):
+// the buffers a lane otherwise gets from hipMalloc -- packed input planes, three
+// activation planes, V and M -- for up to kStaticMaxBatch positions of a net with up
+// to kStaticMaxFp filters (padded count) in the wider storage type (fp32):
+//   V, M   2 x 36 x 256 x 256 x 4 B = 18 874 368
+//   act0   8 x 361 x 64 x 4 B       =    739 328
+//   act[3] 3 x 8 x 361 x 256 x 4 B  =  8 871 936      total 28 485 632 B (27.2 MiB)
+// Every GPU the library runs on holds its own copy from module load to process end.
+// In host code `scratch` is only a handle for hipGetSymbolAddress: the address kernels
+// may use is the one resolved per device in static_scratch().
+constexpr int kStaticMaxBatch = 8;
+constexpr int kStaticMaxFp = 256;
+constexpr int kStaticTp = 256;   // 8 x 25 tiles rounded up to kTileRowPad
+constexpr size_t kStaticTileBytes = (size_t)kPos * kStaticTp * kStaticMaxFp * 4;
+constexpr size_t kStaticAct0Bytes = (size_t)kStaticMaxBatch * kPts * 64 * 4;
+constexpr size_t kStaticActBytes = (size_t)kStaticMaxBatch * kPts * kStaticMaxFp * 4;
+constexpr size_t kStaticBytes = 2 * kStaticTileBytes + kStaticAct0Bytes + 3 * kStaticActBytes;
+static_assert(kStaticTileBytes % 256 == 0 && kStaticAct0Bytes % 256 == 0 &&
+              kStaticActBytes % 256 == 0, "sub-buffers keep the 256-byte alignment");
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of this device's copy of `scratch`; resolved once per device, with
+// that device current (called from the pipe's constructor, i.e. from lzhip_create).
+static unsigned char* static_scratch(int device) {
+    if (device < 0 || device >= kMaxDevices) throw std::invalid_argument("device ordinal out of range");
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        HIP_CHECK(hipSetDevice(device));
+        unsigned char* ptr = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+        if (!ptr) throw std::runtime_error("hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[device] = ptr;
+    }
+    return g_scratch_ptr[device];
+}
+
 template <typename T> struct DevBuf {
     T* p = nullptr;
     size_t count = 0;
@@ -89,7 +129,8 @@ public:
         // Small batches leave more of the device idle at every kernel boundary: a third
         // lane pays up to batch 32 (+10 %) and no longer at 64 (-2 %).
         m_n_lanes = max_batch <= 32 ? 3 : 2;
-        for (int i = 0; i < m_n_lanes; i++) HIP_CHECK(hipStreamCreate(&m_lane[i].stream));
+        // Every refusal comes before the first stream, event or allocation is made: a
+        // constructor that throws runs no destructor.
         m_Fp = round_up(filters, 64);
         if (!gemm_supports_channels<P>(m_Fp))
             throw std::invalid_argument(
@@ -101,6 +142,13 @@ public:
         if ((size_t)kPos * m_Tp * m_Fp * sizeof(P) >= ((size_t)1 << 31))
             throw std::invalid_argument(
                 "max_batch x filters too large: the Winograd tile buffers would exceed 2 GiB");
+        m_static = static_scratch(device);
+        struct Unwind {   // releases what the body below has created if it throws
+            HIPPipeImpl* self;
+            bool armed = true;
+            ~Unwind() { if (armed) self->release_device_objects(); }
+        } unwind{this};
+        for (int i = 0; i < m_n_lanes; i++) HIP_CHECK(hipStreamCreate(&m_lane[i].stream));
         const size_t B = (size_t)max_batch;
         m_din.alloc(B * kInPlanes * kPts);
         m_dpol.alloc(B * 2 * kPts);
@@ -128,9 +176,14 @@ public:
             HIP_CHECK(hipEventCreate(&m_ev_start[i]));
             HIP_CHECK(hipEventCreate(&m_ev_stop[i]));
         }
+        unwind.armed = false;
     }
 
-    ~HIPPipeImpl() override {
+    ~HIPPipeImpl() override { release_device_objects(); }
+
+    // Streams and events (the buffers free themselves).  Also run by the constructor
+    // when it fails half way.
+    void release_device_objects() {
         (void)hipSetDevice(m_device);
         for (auto& ln : m_lane)
             if (ln.stream) (void)hipStreamSynchronize(ln.stream);
@@ -138,11 +191,16 @@ public:
         for (int i = 0; i < kTimerPool; i++) {
             if (m_ev_start[i]) (void)hipEventDestroy(m_ev_start[i]);
             if (m_ev_stop[i]) (void)hipEventDestroy(m_ev_stop[i]);
+            m_ev_start[i] = m_ev_stop[i] = nullptr;
         }
-        for (auto& sl : m_slot)
+        for (auto& sl : m_slot) {
             if (sl.done) (void)hipEventDestroy(sl.done);
-        for (auto& ln : m_lane)
+            sl.done = nullptr;
+        }
+        for (auto& ln : m_lane) {
             if (ln.stream) (void)hipStreamDestroy(ln.stream);
+            ln.stream = nullptr;
+        }
     }
 
     int max_batch() const override { return m_max_batch; }
@@ -210,6 +268,40 @@ public:
         check_ready(n);
         HIP_CHECK(hipSetDevice(m_device));
         run_forward(ln, n, d_in, nullptr, d_pol, d_val);
+        HIP_CHECK(hipGetLastError());
+    }
+
+    // The same forward with every working buffer taken from the device's static
+    // `scratch` array instead of the lane's allocations: kernel launches only, no
+    // allocation of any kind.  Enqueued on lane 0's stream.  All calls on one GPU share
+    // the array (whatever the handle), so calls that overlap on that GPU race; calls on
+    // one handle are ordered by the stream.  Nothing in the array has to start at zero:
+    // every element a kernel reads for a real tile is written earlier in the same call
+    // (rows of V past the last tile feed only rows of M that no kernel reads).
+    void forward_device_static(int n, const float* d_in, float* d_pol, float* d_val) override {
+        Lane& ln = m_lane[0];
+        std::lock_guard<std::mutex> lk(ln.mu);
+        if (m_layers.empty()) throw std::invalid_argument("push_weights has not been called");
+        if (n < 1 || n > kStaticMaxBatch || n > m_max_batch)
+            throw std::invalid_argument(
+                "the no-allocation forward takes 1..8 positions (and at most max_batch): its "
+                "static working memory is sized for 8");
+        if (m_Fp > kStaticMaxFp)
+            throw std::invalid_argument(
+                "the no-allocation forward takes networks of up to 256 filters: its static "
+                "working memory is sized for that");
+        HIP_CHECK(hipSetDevice(m_device));
+        unsigned char* base = m_static;
+        Work w;
+        w.stream = ln.stream;
+        w.Tp = kStaticTp;
+        w.V = reinterpret_cast<P*>(base);
+        w.M = reinterpret_cast<P*>(base + kStaticTileBytes);
+        w.act0 = reinterpret_cast<P*>(base + 2 * kStaticTileBytes);
+        for (int i = 0; i < 3; i++)
+            w.act[i] = reinterpret_cast<P*>(base + 2 * kStaticTileBytes + kStaticAct0Bytes +
+                                            (size_t)i * kStaticActBytes);
+        enqueue_forward(w, n, d_in, nullptr, d_pol, d_val, false);
         HIP_CHECK(hipGetLastError());
     }
 
@@ -475,6 +567,24 @@ private:
     };
     static constexpr int kLanes = 3;   // upper bound; m_n_lanes are in use
 
+    // The working buffers of one forward as plain pointers: a lane's own allocations
+    // or the static array.  Tp = rows of V and M per Winograd position.
+    struct Work {
+        hipStream_t stream = nullptr;
+        P *act0 = nullptr, *act[3] = {nullptr, nullptr, nullptr}, *V = nullptr, *M = nullptr;
+        int Tp = 0;
+    };
+    Work work_of(Lane& ln) const {
+        Work w;
+        w.stream = ln.stream;
+        w.act0 = ln.act0.p;
+        for (int i = 0; i < 3; i++) w.act[i] = ln.act[i].p;
+        w.V = ln.V.p;
+        w.M = ln.M.p;
+        w.Tp = m_Tp;
+        return w;
+    }
+
     struct Layer {
         int C = 0, Cp = 0;
         DevBuf<P> U;
@@ -567,33 +677,36 @@ private:
     // output), and by the last layer for the 1x1 heads.
     void enqueue_forward(Lane& ln, int n, const float* d_in, const uint32_t* d_bits,
                          float* d_pol, float* d_val, bool timed) {
+        enqueue_forward(work_of(ln), n, d_in, d_bits, d_pol, d_val, timed);
+    }
+    void enqueue_forward(const Work& w, int n, const float* d_in, const uint32_t* d_bits,
+                         float* d_pol, float* d_val, bool timed) {
         const int nl = (int)m_layers.size();
         const int Tu = n * kTilesPerBoard;
         if (d_in)
-            launch_pack_input<P>(d_in, ln.act0.p, n, kInPlanes, m_C0p, ln.stream,
+            launch_pack_input<P>(d_in, w.act0, n, kInPlanes, m_C0p, w.stream,
                                  timer(timed, LZHIP_K_PACK));
         else
-            launch_pack_input_bits<P>(d_bits, ln.act0.p, n, kInPlanes, m_C0p, ln.stream,
+            launch_pack_input_bits<P>(d_bits, w.act0, n, kInPlanes, m_C0p, w.stream,
                                       timer(timed, LZHIP_K_PACK));
-        launch_in_transform<P>(ln.act0.p, ln.V.p, n, m_C0p, m_Tp, ln.stream,
-                               timer(timed, LZHIP_K_IN));
+        launch_in_transform<P>(w.act0, w.V, n, m_C0p, w.Tp, w.stream, timer(timed, LZHIP_K_IN));
         int cur = 0, nxt = 1;  // block input (skip) / block output
         for (int l = 0; l < nl; l++) {
             Layer& L = m_layers[l];
-            launch_gemm<P>(ln.V.p, L.U.p, ln.M.p, Tu, m_Tp, L.Cp, m_Fp, ln.stream,
+            launch_gemm<P>(w.V, L.U.p, w.M, Tu, w.Tp, L.Cp, m_Fp, w.stream,
                            timer(timed, LZHIP_K_GEMM));
             const bool block_end = (l % 2) == 0;      // layer 0 and second convs
-            const P* res = (block_end && l >= 2) ? ln.act[cur].p : nullptr;
-            P* out = l == 0 ? ln.act[cur].p : ln.act[nxt].p;
+            const P* res = (block_end && l >= 2) ? w.act[cur] : nullptr;
+            P* out = l == 0 ? w.act[cur] : w.act[nxt];
             if (l == nl - 1) {
-                launch_out_transform<P>(ln.M.p, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n,
-                                        m_Fp, m_Tp, ln.stream, timer(timed, LZHIP_K_OUT));
-                launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, ln.stream,
+                launch_out_transform<P>(w.M, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp,
+                                        w.Tp, w.stream, timer(timed, LZHIP_K_OUT));
+                launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, w.stream,
                                     timer(timed, LZHIP_K_HEAD));
             } else {
-                launch_out_in_transform<P>(ln.M.p, res, block_end ? out : nullptr, ln.V.p,
-                                           L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, m_Tp,
-                                           ln.stream, timer(timed, LZHIP_K_OUTIN));
+                launch_out_in_transform<P>(w.M, res, block_end ? out : nullptr, w.V, L.d_scale.p,
+                                           L.d_mean.p, L.rfac, n, m_Fp, w.Tp, w.stream,
+                                           timer(timed, LZHIP_K_OUTIN));
             }
             if (block_end && l >= 2) { const int o = cur; cur = nxt; nxt = o; }
         }
@@ -683,6 +796,7 @@ private:
     static constexpr int kTimerPool = 512;
     int m_device, m_max_batch, m_filters;
     int m_Fp = 0, m_C0p = 0, m_Tp = 0;
+    unsigned char* m_static = nullptr;   // this device's copy of the static working memory
     Lane m_lane[kLanes];
     int m_n_lanes = 2;
     DevBuf<float> m_din, m_dpol, m_dval, m_w3, m_scalar;  // evaluate_batch / calibration
