@@ -240,6 +240,16 @@ public:
                 }
             L.U.alloc(tmp.size());
             HIP_CHECK(hipMemcpy(L.U.p, tmp.data(), tmp.size() * sizeof(P), hipMemcpyHostToDevice));
+            // Second copy in the fragment order of the streaming GEMM, where the largest
+            // batch of this handle can take that kernel.
+            if constexpr (sizeof(P) == 2) {
+                if (gemm_stream_shape(m_max_batch * kTilesPerBoard, L.Cp, m_Fp)) {
+                    build_stream_filters(U[l], L.C, F, L.Cp, m_Fp, tmp.data());
+                    L.Uf.alloc(tmp.size());
+                    HIP_CHECK(hipMemcpy(L.Uf.p, tmp.data(), tmp.size() * sizeof(P),
+                                        hipMemcpyHostToDevice));
+                }
+            }
             L.mean.assign(bn_mean[l], bn_mean[l] + F);
             L.scale.assign(bn_scale[l], bn_scale[l] + F);
             L.d_mean.alloc(m_Fp);
@@ -496,7 +506,7 @@ public:
         HIP_CHECK(hipMemcpy(d_sc.p, sc.data(), sizeof(float) * m_Fp, hipMemcpyHostToDevice));
         HIP_CHECK(hipMemcpy(d_mn.p, mn.data(), sizeof(float) * m_Fp, hipMemcpyHostToDevice));
         launch_in_transform<P>(a_in, ln.V.p, n, Cp, m_Tp, ln.stream, nullptr);
-        launch_gemm<P>(ln.V.p, L.U.p, ln.M.p, Tu, m_Tp, Cp, m_Fp, ln.stream, nullptr);
+        launch_gemm<P>(ln.V.p, L.U.p, L.Uf.p, ln.M.p, Tu, m_Tp, Cp, m_Fp, ln.stream, nullptr);
         launch_out_transform<P>(ln.M.p, r, ln.act[2].p, d_sc.p, d_mn.p, 1.0f, n, m_Fp, m_Tp,
                                 ln.stream, nullptr);
         HIP_CHECK(hipGetLastError());
@@ -588,6 +598,7 @@ private:
     struct Layer {
         int C = 0, Cp = 0;
         DevBuf<P> U;
+        DevBuf<P> Uf;                         // fragment order (streaming GEMM), may be empty
         std::vector<float> mean, scale;       // as pushed (unscaled)
         DevBuf<float> d_mean, d_scale;        // with activation scales folded in
         float rfac = 1.0f;
@@ -628,7 +639,7 @@ private:
         Layer& L = m_layers[l];
         const int Tu = n * kTilesPerBoard;
         launch_in_transform<P>(in, ln.V.p, n, L.Cp, m_Tp, ln.stream, timer(timed, LZHIP_K_IN));
-        launch_gemm<P>(ln.V.p, L.U.p, ln.M.p, Tu, m_Tp, L.Cp, m_Fp, ln.stream,
+        launch_gemm<P>(ln.V.p, L.U.p, L.Uf.p, ln.M.p, Tu, m_Tp, L.Cp, m_Fp, ln.stream,
                        timer(timed, LZHIP_K_GEMM));
         launch_out_transform<P>(ln.M.p, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, m_Tp,
                                 ln.stream, timer(timed, LZHIP_K_OUT));
@@ -693,7 +704,7 @@ private:
         int cur = 0, nxt = 1;  // block input (skip) / block output
         for (int l = 0; l < nl; l++) {
             Layer& L = m_layers[l];
-            launch_gemm<P>(w.V, L.U.p, w.M, Tu, w.Tp, L.Cp, m_Fp, w.stream,
+            launch_gemm<P>(w.V, L.U.p, L.Uf.p, w.M, Tu, w.Tp, L.Cp, m_Fp, w.stream,
                            timer(timed, LZHIP_K_GEMM));
             const bool block_end = (l % 2) == 0;      // layer 0 and second convs
             const P* res = (block_end && l >= 2) ? w.act[cur] : nullptr;

@@ -1370,6 +1370,246 @@ __global__ __launch_bounds__(512) void wino_gemm_split_k(const P* __restrict__ V
     }
 }
 
+// ---------------------------------------------------------------------------
+// Filter-stationary streaming GEMM (fp16 storage).  One work-group of 8 wavefronts
+// owns one Winograd position and a run of consecutive 32-row blocks of V; wavefront
+// w owns output channels 32w..32w+31 of a 256-channel column tile and keeps its
+// share of U_p -- 32 channels x Cp input channels -- in registers for the whole
+// kernel (Cp/4 registers per lane), already in the order the matrix instruction
+// wants it.  V streams through: a 32-row block (all Cp input channels, so the
+// contraction of those rows completes in one step) is requested kStreamAhead steps
+// ahead into registers and passes through a three-stage LDS ring, where all eight
+// wavefronts read it as their column operand.  A step multiplies one block; the
+// fragment reads of the block's second half and of the next block's first half are
+// issued ahead of the matrix instructions that hide them, and one barrier ends the
+// step.  Loads of later blocks, matrix instructions and stores of earlier blocks are
+// in flight together from the first block to the last.
+//
+// Output: register r of lane l of a 32x32 accumulator holds row 8(r/4) + 4(l/32) + r%4
+// of the row operand.  The row operand is U, and the host stores U's channels permuted
+// (gemm_stream_channel) so that this lane's sixteen registers are the channels
+// 16(r/8) + 8(l/32) + r%8 of the wavefront's 32, i.e. two 16-byte runs.  Those go into
+// an LDS copy of the block's 32 x 256 result, and one step later (behind the barrier
+// that is there anyway) every wavefront sends four whole rows of it, 1 KiB per store
+// instruction.  The stores are write-through (sc0 sc1): whole lines leave for memory
+// while the kernel runs, instead of collecting as dirty lines in the L2 that the end
+// of the kernel has to flush with nothing else in flight (measured at 64 boards and
+// 256 filters: 14.2 -> 12.3 us per launch; in 32-byte pieces straight from the
+// accumulators write-through is slower than write-back).
+//
+// Uf layout ("fragment order"): [36][Kp/32][Cp/16][64 lanes][8 halves]; lane l of
+// fragment (p, wb, kc) holds U_p[32 wb + gemm_stream_channel(l % 32)][16 kc + 8 (l / 32) + 0..7],
+// so every operand load of a wavefront is one contiguous KiB.
+constexpr int kStreamBlocks = 8;   // 32-row blocks per work-group (steps of the pipeline)
+constexpr int kStreamAhead = 2;    // blocks requested ahead of the one being multiplied
+constexpr int kStoreThrough = 17;  // cache policy of a raw buffer store: sc0 | sc1 (write-through)
+
+__host__ __device__ constexpr int gemm_stream_channel(int i) {
+    // i = 8q + 4h + e  ->  16 (q / 2) + 8 h + 4 (q % 2) + e
+    return 16 * (i >> 4) + 8 * ((i >> 2) & 1) + 4 * ((i >> 3) & 1) + (i & 3);
+}
+
+template <int NKC>
+__global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restrict__ V,
+                                                          const half_t* __restrict__ Uf,
+                                                          half_t* __restrict__ M, int T, int Tp,
+                                                          int Kp, int chunks, int nblk_total,
+                                                          int tiles_n, int seg) {
+    constexpr int NBLK = kStreamBlocks, D = kStreamAhead;
+    constexpr int Cp = NKC * 16;
+    constexpr int HK = NKC / 2;                  // fragments per half block
+    constexpr int CPRW = Cp / 8;                 // 16-byte chunks per row
+    constexpr int NCH = 32 * CPRW;               // chunks per block
+    constexpr int CH = (NCH + 511) / 512;        // chunk loads per thread and block
+    constexpr bool FULL = NCH % 512 == 0;        // every thread has all CH chunks
+    constexpr int ROWE = Cp + 8;                 // padded LDS row (halves): conflict-free 16-byte reads
+    constexpr int STAGE = 32 * ROWE;
+    constexpr int OROW = 256 + 8;                // row of the output copy (halves)
+    constexpr int OSTAGE = 32 * OROW;
+    static_assert(NKC % 2 == 0 && D == 2, "pipeline shape");
+
+    __shared__ __attribute__((aligned(16))) half_t smem[3 * STAGE + 2 * OSTAGE];
+    half_t* const obuf = smem + 3 * STAGE;
+
+    const int n_items = kPos * chunks * tiles_n;
+    const int xcd = blockIdx.x & 7;
+    const int item = xcd * seg + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= seg || item >= n_items) return;
+    const int tn = item % tiles_n;
+    const int rest = item / tiles_n;
+    const int ch = rest % chunks;
+    const int p = rest / chunks;
+    // this work-group's real blocks: [blk0, blk1), at most NBLK of them
+    const int blk0 = (ch * nblk_total) / chunks;
+    const int blk1 = ((ch + 1) * nblk_total) / chunks;
+    const int nreal = blk1 - blk0;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hh = lane >> 5, jrow = lane & 31;
+
+    // chunk coordinates of this thread's loads within a block
+    int lrow[CH], lcc[CH];
+    bool lval[CH];
+#pragma unroll
+    for (int i = 0; i < CH; i++) {
+        const int idx = tid + i * 512;
+        lval[i] = FULL || idx < NCH;
+        lrow[i] = (idx / CPRW) & 31;
+        lcc[i] = idx % CPRW;
+    }
+    const half_t* Vp = V + (size_t)p * Tp * Cp;
+
+    int4v st[D][CH];
+    auto gload = [&](int slot, int s) {
+        // steps past the last real block re-read that block (cache hits, never stored)
+        const int blk = blk0 + (s < nreal ? s : nreal - 1);
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int row = min(blk * 32 + lrow[i], T - 1);
+            if (lval[i])
+                st[slot][i] =
+                    *reinterpret_cast<const int4v*>(Vp + (size_t)row * Cp + lcc[i] * 8);
+        }
+    };
+    auto lstore = [&](int slot, int buf) {
+        half_t* S = smem + buf * STAGE;
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+            if (lval[i]) *reinterpret_cast<int4v*>(&S[lrow[i] * ROWE + lcc[i] * 8]) = st[slot][i];
+    };
+
+    // This wavefront's share of U, then the first two blocks of V.
+    int4v u[NKC];
+    {
+        const half_t* Up =
+            Uf + ((((size_t)p * (Kp / 32) + (size_t)tn * 8 + wave) * NKC) * 64 + lane) * 8;
+#pragma unroll
+        for (int kc = 0; kc < NKC; kc++)
+            u[kc] = *reinterpret_cast<const int4v*>(Up + (size_t)kc * 64 * 8);
+    }
+    gload(0, 0);
+    gload(1, 1);
+    lstore(0, 0);
+    lstore(1, 1);
+    __syncthreads();
+
+    // M goes out through a raw buffer whose extent is the T real rows of this position:
+    // rows past the last tile, and the steps past this work-group's last block, get an
+    // offset outside it and are dropped by the hardware, so the stores are unconditional
+    // straight-line code (a branch around them would make the compiler wait for every
+    // outstanding load behind it).
+    const size_t m_bytes = (size_t)T * Kp * sizeof(half_t);
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(M + (size_t)p * Tp * Kp, m_bytes);
+    const unsigned m_rowb = (unsigned)Kp * 2u;
+    const unsigned m_col = (unsigned)(tn * 256 + jrow * 8) * 2u;
+    // wavefront w sends rows 4w..4w+3 of a block: two whole rows per store instruction
+    auto send_rows = [&](int s) {
+        const half_t* O = obuf + (s & 1) * OSTAGE;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int r = wave * 4 + hh + 2 * i;
+            const int4v v = *reinterpret_cast<const int4v*>(O + r * OROW + jrow * 8);
+            const unsigned row = (unsigned)((blk0 + s) * 32 + r);
+            const unsigned vo = s < nreal ? row * m_rowb + m_col : 0x7ffffff0u;
+            __builtin_amdgcn_raw_buffer_store_b128(v, rM, vo, 0, kStoreThrough);
+        }
+    };
+
+    const int frag = jrow * ROWE + hh * 8;
+    int4v alo[HK], ahi[HK];
+#pragma unroll
+    for (int kc = 0; kc < HK; kc++) alo[kc] = *reinterpret_cast<const int4v*>(smem + frag + kc * 16);
+
+#pragma unroll
+    for (int s = 0; s < NBLK; s++) {
+        if (s + D < NBLK) gload(s % D, s + D);
+        if (s > 0) send_rows(s - 1);
+        const half_t* S = smem + (s % 3) * STAGE + frag;
+#pragma unroll
+        for (int kc = 0; kc < HK; kc++)
+            ahi[kc] = *reinterpret_cast<const int4v*>(S + (HK + kc) * 16);
+        __builtin_amdgcn_sched_barrier(0);
+        float16v acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+#pragma unroll
+        for (int kc = 0; kc < HK; kc++)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, u[kc]),
+                                                         __builtin_bit_cast(half8v, alo[kc]), acc,
+                                                         0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + 1 < NBLK) {
+            const half_t* Sn = smem + ((s + 1) % 3) * STAGE + frag;
+#pragma unroll
+            for (int kc = 0; kc < HK; kc++)
+                alo[kc] = *reinterpret_cast<const int4v*>(Sn + kc * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kc = 0; kc < HK; kc++)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8v, u[HK + kc]),
+                                                         __builtin_bit_cast(half8v, ahi[kc]), acc,
+                                                         0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + 2 < NBLK) lstore((s + 2) % D, (s + 2) % 3);
+        half8v o0, o1;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            o0[e] = to_storage<half_t>(acc[e]);
+            o1[e] = to_storage<half_t>(acc[8 + e]);
+        }
+        half_t* O = obuf + (s & 1) * OSTAGE + jrow * OROW + wave * 32 + hh * 8;
+        *reinterpret_cast<half8v*>(O) = o0;
+        *reinterpret_cast<half8v*>(O + 16) = o1;
+        __syncthreads();
+    }
+    send_rows(NBLK - 1);
+}
+
+// Fragment-order copy of one layer's filters for wino_gemm_stream_k, built on the host:
+// src is the reference layout [36][C][F] (F fastest), dst [36][Kp/32][Cp/16][64][8].
+void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, half_t* dst) {
+    const int nkc = Cp / 16, nwb = Kp / 32;
+    for (int p = 0; p < kPos; p++)
+        for (int wb = 0; wb < nwb; wb++)
+            for (int kc = 0; kc < nkc; kc++)
+                for (int l = 0; l < 64; l++) {
+                    const int k = 32 * wb + gemm_stream_channel(l & 31);
+                    for (int e = 0; e < 8; e++) {
+                        const int c = 16 * kc + 8 * (l >> 5) + e;
+                        float v = 0.0f;
+                        if (c < C && k < F) v = src[((size_t)p * C + c) * F + k];
+                        dst[((((size_t)p * nwb + wb) * nkc + kc) * 64 + l) * 8 + e] = (half_t)v;
+                    }
+                }
+}
+
+// Whether launch_gemm would take the streaming kernel for this shape (the caller then has
+// to hold the fragment-order filters).
+bool gemm_stream_shape(int T, int Cp, int Kp) {
+    if (Kp % 256 != 0 || !(Cp == 64 || Cp == 256)) return false;
+    const int nblk = (T + 31) / 32;
+    const int chunks = (nblk + kStreamBlocks - 1) / kStreamBlocks;
+    return kPos * chunks * (Kp / 256) >= 200;
+}
+
+static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
+                               int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
+    const int nblk = (T + 31) / 32;
+    const int chunks = (nblk + kStreamBlocks - 1) / kStreamBlocks;
+    const int tiles_n = Kp / 256;
+    const int n_items = kPos * chunks * tiles_n;
+    int seg = (n_items + 7) / 8;
+    seg = (seg + tiles_n - 1) / tiles_n * tiles_n;
+    if (Cp == 256)
+        launch(wino_gemm_stream_k<16>, dim3(8 * seg), dim3(512), s, t, V, Uf, M, T, Tp, Kp,
+               chunks, nblk, tiles_n, seg);
+    else
+        launch(wino_gemm_stream_k<4>, dim3(8 * seg), dim3(512), s, t, V, Uf, M, T, Tp, Kp,
+               chunks, nblk, tiles_n, seg);
+}
+
 template <typename P, int NK>
 static void launch_gemm_big(const P* V, const P* U, P* M, int T, int tiles_m, int Tp, int Cp,
                             int Kp, hipStream_t s, LaunchTimer* t) {
@@ -1405,10 +1645,16 @@ template bool gemm_supports_channels<half_t>(int);
 // T = number of real tile rows (25 per board); Tp (the row count of V and M)
 // must be a multiple of 256.
 template <typename P>
-void launch_gemm(const P* V, const P* U, P* M, int T, int Tp, int Cp, int Kp, hipStream_t s,
-                 LaunchTimer* t) {
+void launch_gemm(const P* V, const P* U, const P* Uf, P* M, int T, int Tp, int Cp, int Kp,
+                 hipStream_t s, LaunchTimer* t) {
     constexpr int BK = 128 / (int)sizeof(P);
     const int nk = Cp / BK;
+    if constexpr (sizeof(P) == 2) {
+        if (Uf != nullptr && gemm_stream_shape(T, Cp, Kp)) {
+            launch_gemm_stream(V, Uf, M, T, Tp, Cp, Kp, s, t);
+            return;
+        }
+    }
     // The 256 x 256 tile pays off once its tiles can occupy most of the 256 compute units
     // (measured at 256 filters: from 6 row tiles = 216 work-groups, batch 52; with 5 = 180 the
     // 128 x 128 tiles are 2 % ahead; fp32 keeps the earlier hand-over at 160).
@@ -1661,8 +1907,8 @@ void launch_heads(const float* pol, const float* val, HeadParams hp, float tempe
                                             LaunchTimer*);                                     \
     template void launch_in_transform<P>(const P*, P*, int, int, int, hipStream_t,             \
                                          LaunchTimer*);                                        \
-    template void launch_gemm<P>(const P*, const P*, P*, int, int, int, int, hipStream_t,      \
-                                 LaunchTimer*);                                                \
+    template void launch_gemm<P>(const P*, const P*, const P*, P*, int, int, int, int,         \
+                                 hipStream_t, LaunchTimer*);                                   \
     template void launch_out_transform<P>(const P*, const P*, P*, const float*, const float*,  \
                                           float, int, int, int, hipStream_t, LaunchTimer*);    \
     template void launch_out_in_transform<P>(const P*, const P*, P*, P*, const float*,         \
