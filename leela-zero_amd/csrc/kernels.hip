@@ -20,6 +20,7 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 
 #define SQ2 1.4142135623730951f
+constexpr int kStoreThrough = 17;  // cache policy of a raw buffer store: sc0 | sc1 (write-through)
 
 // ---------------------------------------------------------------------------
 // Per-lane channel vector: how many consecutive channels one lane owns in the
@@ -73,18 +74,17 @@ __device__ __forceinline__ void bt6(const float i0, const float i1, const float 
     o5 = i1 + i3 * (-5.0f / 2.0f) + i5;
 }
 
-// o = A^T i for one 6-vector (reference src/CPUPipe.cpp:225-238).
+// o = A^T i for one 6-vector (reference src/CPUPipe.cpp:225-238; the same sums,
+// associated so that they take twelve operations).
 __device__ __forceinline__ void at6(const float i0, const float i1, const float i2,
                                     const float i3, const float i4, const float i5, float& o0,
                                     float& o1, float& o2, float& o3) {
-    const float t1p2 = (i1 + i2) * (1.0f / 2.0f);
-    const float t1m2 = (i1 - i2) * (SQ2 / 4.0f);
-    const float t3p4 = i3 + i4;
-    const float t3m4 = (i3 - i4) * SQ2;
-    o0 = i0 + t1p2 + t1p2 + t3p4;
-    o1 = t1m2 + t1m2 + t3m4;
-    o2 = t1p2 + t3p4 + t3p4;
-    o3 = t1m2 + t3m4 + t3m4 + i5;
+    const float s12 = i1 + i2, d12 = i1 - i2;
+    const float s34 = i3 + i4, d34 = i3 - i4;
+    o0 = (i0 + s12) + s34;
+    o1 = fmaf(d34, SQ2, d12 * (SQ2 / 2.0f));
+    o2 = fmaf(s34, 2.0f, s12 * 0.5f);
+    o3 = fmaf(d34, 2.0f * SQ2, fmaf(d12, SQ2 / 4.0f, i5));
 }
 
 // ---------------------------------------------------------------------------
@@ -438,17 +438,14 @@ template <> __device__ __forceinline__ half_t act_to_storage<half_t>(float v) {
 // arithmetic of the one compute unit a workgroup runs on, and 32 or 16 channels
 // per workgroup (4 or 8 tiles per wavefront, 7 or 4 wavefronts) spread a board
 // over more compute units.
-// Cache policy of the fused transform's stores: write-through (sc0 sc1).  Every store
-// instruction writes whole 128-byte lines (64 channels of one tile row or board point), and
-// nothing in this kernel reads them again: written through, they leave for memory while the
-// kernel runs instead of staying behind as dirty lines that the end of the kernel has to
-// flush (measured at 64 boards, 256 filters: 15.2 -> 14.0 us per launch).
-#ifndef LZ_XA
-#define LZ_XA 17
-#endif
-#ifndef LZ_XV
-#define LZ_XV 17
-#endif
+// Cache policy of the fused transform's stores.  With 64 channels per work-group every
+// store instruction writes whole 128-byte lines (64 channels of one tile row or board
+// point), and nothing in the kernel reads them again: written through (sc0 sc1) they leave
+// for memory while the kernel runs instead of staying behind as dirty lines that the end
+// of the kernel has to flush (measured at 64 boards, 256 filters: 15.2 -> 14.0 us per
+// launch).  The narrower work-groups write half and quarter lines, which written through
+// cost twice the time (32 channels at 64 boards: 16.4 us against 12.9): they stay write-back.
+template <int CG> constexpr int xform_store_policy() { return CG == 64 ? kStoreThrough : 0; }
 constexpr int kPlane = 22;       // LDS plane: 19 points + 1 zero halo before + 2 after
 constexpr int fuse_waves(int cg) { return (kTilesPerBoard + 128 / cg - 1) / (128 / cg); }
 
@@ -493,11 +490,11 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     const unsigned soff_t =
         ((unsigned)(b * kTilesPerBoard + TPW * wave) * (unsigned)Kp + cg * CG) * esz;
     const unsigned soff_a = ((unsigned)(b * kPts) * (unsigned)Kp + cg * CG) * esz;
-    float sc[2], mn[2];
+    float sc[2], nb[2];   // scale * (y - mean) = y * scale + nb
 #pragma unroll
     for (int v = 0; v < 2; v++) {
         sc[v] = bn_scale[cg * CG + cl * 2 + v];
-        mn[v] = bn_mean[cg * CG + cl * 2 + v];
+        nb[v] = -sc[v] * bn_mean[cg * CG + cl * 2 + v];
     }
 
     // All loads of the pass go out before any arithmetic.  M's go first, column by
@@ -587,10 +584,10 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
 #pragma unroll
             for (int jj = 0; jj < 4; jj++) {
                 pair_t sv;
-                sv.x = act_to_storage<P>(
-                    fmaxf(0.0f, sc[0] * (o[0][i * 4 + jj] - mn[0]) + rfac * (float)r[i * 4 + jj].x));
-                sv.y = act_to_storage<P>(
-                    fmaxf(0.0f, sc[1] * (o[1][i * 4 + jj] - mn[1]) + rfac * (float)r[i * 4 + jj].y));
+                sv.x = act_to_storage<P>(fmaxf(
+                    0.0f, fmaf((float)r[i * 4 + jj].x, rfac, fmaf(o[0][i * 4 + jj], sc[0], nb[0]))));
+                sv.y = act_to_storage<P>(fmaxf(
+                    0.0f, fmaf((float)r[i * 4 + jj].y, rfac, fmaf(o[1][i * 4 + jj], sc[1], nb[1]))));
                 keep[i * 4 + jj] = sv;
                 if (valid && i < ny && jj < nx) origin[((i + 1) * kPlane + (jj + 1)) * CP] = sv;
             }
@@ -605,7 +602,7 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
 #pragma unroll
             for (int jj = 0; jj < 4; jj++)
                 if (valid && i < ny && jj < nx)
-                    BufIO2<P>::template store<LZ_XA>(keep[i * 4 + jj], rA, voff_a,
+                    BufIO2<P>::template store<xform_store_policy<CG>()>(keep[i * 4 + jj], rA, voff_a,
                                      soff_a + (unsigned)(i * kBoard + jj) * (unsigned)Kp * esz);
     }
 
@@ -641,7 +638,7 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
             unsigned so = soff_t;
 #pragma unroll
             for (int p = 0; p < 36; p++) {
-                BufIO2<P>::template store<LZ_XV>(outp[p], rV, voff_t, so);
+                BufIO2<P>::template store<xform_store_policy<CG>()>(outp[p], rV, voff_t, so);
                 so += pstride;
             }
         }
@@ -1413,22 +1410,21 @@ __global__ __launch_bounds__(512) void wino_gemm_split_k(const P* __restrict__ V
 // Uf layout ("fragment order"): [36][Kp/32][Cp/16][64 lanes][8 halves]; lane l of
 // fragment (p, wb, kc) holds U_p[32 wb + gemm_stream_channel(l % 32)][16 kc + 8 (l / 32) + 0..7],
 // so every operand load of a wavefront is one contiguous KiB.
-constexpr int kStreamBlocks = 8;   // 32-row blocks per work-group (steps of the pipeline)
+constexpr int kStreamBlocks = 8;   // most 32-row blocks per work-group (steps of the pipeline)
 constexpr int kStreamAhead = 2;    // blocks requested ahead of the one being multiplied
-constexpr int kStoreThrough = 17;  // cache policy of a raw buffer store: sc0 | sc1 (write-through)
 
 __host__ __device__ constexpr int gemm_stream_channel(int i) {
     // i = 8q + 4h + e  ->  16 (q / 2) + 8 h + 4 (q % 2) + e
     return 16 * (i >> 4) + 8 * ((i >> 2) & 1) + 4 * ((i >> 3) & 1) + (i & 3);
 }
 
-template <int NKC>
+template <int NKC, int NBLK>
 __global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restrict__ V,
                                                           const half_t* __restrict__ Uf,
                                                           half_t* __restrict__ M, int T, int Tp,
                                                           int Kp, int chunks, int nblk_total,
                                                           int tiles_n, int seg) {
-    constexpr int NBLK = kStreamBlocks, D = kStreamAhead;
+    constexpr int D = kStreamAhead;
     constexpr int Cp = NKC * 16;
     constexpr int HK = NKC / 2;                  // fragments per half block
     constexpr int CPRW = Cp / 8;                 // 16-byte chunks per row
@@ -1502,9 +1498,9 @@ __global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restri
             u[kc] = *reinterpret_cast<const int4v*>(Up + (size_t)kc * 64 * 8);
     }
     gload(0, 0);
-    gload(1, 1);
+    if (NBLK > 1) gload(1, 1);
     lstore(0, 0);
-    lstore(1, 1);
+    if (NBLK > 1) lstore(1, 1);
     __syncthreads();
 
     // M goes out through a raw buffer whose extent is the T real rows of this position:
@@ -1598,29 +1594,48 @@ void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, half_t
                 }
 }
 
-// Whether launch_gemm would take the streaming kernel for this shape (the caller then has
-// to hold the fragment-order filters).
-bool gemm_stream_shape(int T, int Cp, int Kp) {
-    if (Kp % 256 != 0 || !(Cp == 64 || Cp == 256)) return false;
+// Blocks per work-group for T tile rows: the fewest (a power of two up to kStreamBlocks)
+// with which one round of work-groups covers the 256 compute units, so that a batch of 8
+// boards runs one block per work-group and 64 boards eight.
+static int gemm_stream_blocks(int T, int Kp) {
     const int nblk = (T + 31) / 32;
-    const int chunks = (nblk + kStreamBlocks - 1) / kStreamBlocks;
-    return kPos * chunks * (Kp / 256) >= 200;
+    const int per_pos = 256 / (kPos * (Kp / 256));           // work-groups per position in one round
+    int nb = 1;
+    while (nb < kStreamBlocks && (nblk + nb - 1) / nb > per_pos) nb *= 2;
+    return nb;
 }
 
-static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
-                               int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
+// Whether launch_gemm takes the streaming kernel for this shape (the caller then has to
+// hold the fragment-order filters): fp16 nets of 256 filters, any batch.
+bool gemm_stream_shape(int T, int Cp, int Kp) {
+    return T >= 1 && Kp == 256 && (Cp == 64 || Cp == 256);
+}
+
+template <int NKC>
+static void launch_gemm_stream_nkc(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
+                                   int Kp, hipStream_t s, LaunchTimer* t) {
     const int nblk = (T + 31) / 32;
-    const int chunks = (nblk + kStreamBlocks - 1) / kStreamBlocks;
+    const int nb = gemm_stream_blocks(T, Kp);
+    const int chunks = (nblk + nb - 1) / nb;
     const int tiles_n = Kp / 256;
     const int n_items = kPos * chunks * tiles_n;
     int seg = (n_items + 7) / 8;
     seg = (seg + tiles_n - 1) / tiles_n * tiles_n;
+    const dim3 grid(8 * seg), block(512);
+    switch (nb) {
+        case 1: launch(wino_gemm_stream_k<NKC, 1>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        case 2: launch(wino_gemm_stream_k<NKC, 2>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        case 4: launch(wino_gemm_stream_k<NKC, 4>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        default: launch(wino_gemm_stream_k<NKC, 8>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+    }
+}
+
+static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
+                               int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
     if (Cp == 256)
-        launch(wino_gemm_stream_k<16>, dim3(8 * seg), dim3(512), s, t, V, Uf, M, T, Tp, Kp,
-               chunks, nblk, tiles_n, seg);
+        launch_gemm_stream_nkc<16>(V, Uf, M, T, Tp, Kp, s, t);
     else
-        launch(wino_gemm_stream_k<4>, dim3(8 * seg), dim3(512), s, t, V, Uf, M, T, Tp, Kp,
-               chunks, nblk, tiles_n, seg);
+        launch_gemm_stream_nkc<4>(V, Uf, M, T, Tp, Kp, s, t);
 }
 
 template <typename P, int NK>

@@ -66,7 +66,7 @@ def test_single_layer_stages(pkg, netgen, orc, precision, filters):
     pipe.close()
 
 
-def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None):
+def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None, all_raw=False):
     """Raw planes, logits, policy and value of the HIP pipe against the oracle.
 
     The reference's answer is itself only defined up to its BLAS back-end's summation
@@ -74,13 +74,24 @@ def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None):
     reach 1e3..1e8, so a last-ulp change of the planes can move a non-saturated
     probability by more than 1e-4.  Each position is therefore also evaluated with the
     oracle's second sgemm provider; where the two oracle runs disagree by more than a
-    fifth of the tolerance, the position is reported as ill-conditioned and compared at
-    10x their disagreement instead.  Raw planes are always compared at the strict
-    relative tolerance."""
+    fifth of the tolerance, the position is reported as ill-conditioned (with the gap
+    between its two largest logits) and compared at 10x their disagreement instead.  At
+    most one position of a case may take that route.  Raw planes and logits are always
+    compared at the strict relative tolerance, for every position checked; with all_raw
+    the raw planes of every position of the batch are (the oracle runs them on all host
+    threads), whatever idx selects for the head outputs."""
     raw_tol = 1e-5 if precision == 0 else 2e-2
     p_tol = 1e-4 if precision == 0 else 2e-2
     policy, value, logits, pol, val = pipe.evaluate_batch(x, want_raw=True)
-    worst = dict(pol=0.0, val=0.0, policy=0.0, value=0.0, ill_conditioned=0)
+    worst = dict(pol=0.0, val=0.0, logits=0.0, policy=0.0, value=0.0, ill_conditioned=0)
+    if all_raw:
+        import os
+        rp_all, rv_all, _ = ref.forward_many(x, threads=min(16, os.cpu_count() or 1))
+        for i in range(x.shape[0]):
+            e_pol, e_val = rel_l2(pol[i], rp_all[i]), rel_l2(val[i], rv_all[i])
+            assert e_pol <= raw_tol and e_val <= raw_tol, ("raw planes", i, e_pol, e_val)
+            worst["pol"] = max(worst["pol"], e_pol)
+            worst["val"] = max(worst["val"], e_val)
     have_blas = orc.use_openblas() != "builtin"
     orc.use_builtin()
     for i in (range(x.shape[0]) if idx is None else idx):
@@ -96,8 +107,15 @@ def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None):
             if noise > p_tol / 5:
                 worst["ill_conditioned"] += 1
                 tol_i = max(p_tol, 10 * noise)
+                top = np.sort(hd["logits"])[-2:]
+                print("ill-conditioned position %d: top-2 logit gap %.4g, oracle back ends "
+                      "differ by %.3g, compared at %.3g" % (i, float(top[1] - top[0]), noise,
+                                                            tol_i), flush=True)
         worst["pol"] = max(worst["pol"], rel_l2(pol[i], rp))
         worst["val"] = max(worst["val"], rel_l2(val[i], rv))
+        e_l = rel_l2(logits[i], hd["logits"])
+        worst["logits"] = max(worst["logits"], e_l)
+        assert e_l <= raw_tol, ("logits", i, e_l)
         e_p = max_abs(policy[i], hd["policy"])
         e_v = abs(float(value[i]) - hd["value"])
         worst["policy"] = max(worst["policy"], e_p)
@@ -106,6 +124,7 @@ def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None):
         assert abs(float(policy[i].sum()) - 1.0) < 1e-4
     print("parity", worst, flush=True)
     assert worst["pol"] <= raw_tol and worst["val"] <= raw_tol, worst
+    assert worst["ill_conditioned"] <= 1, worst
     return worst
 
 
@@ -127,14 +146,14 @@ def test_forward_parity(pkg, netgen, orc, blocks, filters, batch, precision):
 
 
 @pytest.mark.parametrize("precision", [0, 1])
-@pytest.mark.parametrize("batch", [64, 52, 41, 33, 24, 10, 2])
+@pytest.mark.parametrize("batch", [72, 64, 52, 41, 36, 35, 33, 24, 21, 18, 17, 10, 9, 8, 2])
 def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
     """256 filters at batch sizes on both sides of every change of kernel shape (GEMM, fp16:
-    256x256 tiles in two passes from 52 boards, persistent 128x128 tiles from 41, 128x64
-    tiles with permuted LDS rows below; fp32: 256x256 from 41, 128x128 from 21, 128x64 with
-    padded rows below; fused transform: 64 channels per work-group from 33 boards, 32 from 6,
-    16 below), in both precisions, including batches whose tile count is not a multiple of
-    any tile height."""
+    the streaming kernel with 1, 2, 4 and 8 blocks of 32 tile rows per work-group, which
+    change at 9, 18 and 36 boards, and more than one round of work-groups at 72; fp32:
+    256x256 tiles from 41 boards, 128x128 from 21, 128x64 with padded rows below; fused
+    transform: 64 channels per work-group from 33 boards, 32 from 6, 16 below), in both
+    precisions, including batches whose tile count is not a multiple of any tile height."""
     print("case: wide 3x256 b%d precision=%d" % (batch, precision), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 256, 3000, precision, batch)
     x = netgen.synthetic_inputs(batch, seed=batch)
@@ -145,7 +164,8 @@ def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
 @pytest.mark.parametrize("blocks,filters,batch", [(20, 256, 32), (40, 256, 64)])
 def test_forward_parity_deep_fp16(pkg, netgen, orc, blocks, filters, batch):
     """The two large fp16 benchmark configurations (20x256 batch 32, 40x256 batch 64) at full
-    size; the oracle checks three positions of the batch."""
+    size: raw planes of every position of the batch against the oracle, head outputs of
+    three of them."""
     print("case: deep fp16 %dx%d b%d" % (blocks, filters, batch), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, blocks, filters, 2000 + blocks,
                                        pkg.FP16, batch)
@@ -153,7 +173,8 @@ def test_forward_parity_deep_fp16(pkg, netgen, orc, blocks, filters, batch):
     s = pipe.act_scales()
     print("act scales: first %s last %s" % (s[:3], s[-3:]), flush=True)
     assert np.all(s >= 1.0) and np.all(np.log2(s) == np.round(np.log2(s)))
-    check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16, idx=[0, batch // 2, batch - 1])
+    check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16, idx=[0, batch // 2, batch - 1],
+                  all_raw=True)
     pipe.close()
 
 
@@ -475,6 +496,21 @@ def test_error_behaviour_on_device(pkg, netgen):
     p = pkg.HIPScheduler(pkg.FP32, 2, device=99)
     with pytest.raises(pkg.LzhipError):
         p.initialize(64)
+
+
+@pytest.mark.parametrize("filters,batch", [(640, 4), (768, 3), (896, 2), (1024, 12), (1024, 8),
+                                           (384, 28), (128, 30), (192, 52)])
+def test_fp16_widths_on_the_tiled_gemm(pkg, netgen, orc, filters, batch):
+    """fp16 widths served by the tiled GEMM kernels (every width but 256): the widest ones --
+    10, 12, 14 and 16 k-slices, at 1024 filters the one-pass 256x256 tile (from 11 boards)
+    and the 128x64 tile below it -- and narrow nets at batches that take the 128x128
+    persistent and the 128x64 tiles."""
+    print("case: fp16 width %d b%d" % (filters, batch), flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, filters, 5000 + filters, pkg.FP16,
+                                       batch)
+    x = netgen.synthetic_inputs(batch, seed=filters + batch)
+    check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16, idx=[0, batch - 1])
+    pipe.close()
 
 
 @pytest.mark.parametrize("precision", [0, 1])
