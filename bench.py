@@ -3,7 +3,12 @@
 network, fp16 storage / fp32 accumulate, batch 64, on one MI355X.
 
 A step is one forward pass (residual tower + 1x1 heads) over one batch of 64
-synthetic positions that already sit in device memory.  Prints one JSON line.
+synthetic positions that already sit in device memory; `value` is measured over exactly
+--steps such steps.  The same JSON line also carries the rate through host buffers (PCIe
+inside the timed region), the figure repeated over five blocks of --steps forwards, the
+roofline of the GEMM and of the transforms from per-launch device timestamps, what a plain
+copy of the same bytes takes on this box, the CPU baseline, the same network in fp32 and
+the three smaller configurations.
 """
 import argparse
 import json
@@ -21,12 +26,24 @@ PEAK_MFMA_F16 = 2.5e15   # dense fp16 matrix FLOP/s, MI355X
 PEAK_MFMA_F32 = 157.3e12
 PEAK_HBM = 8.0e12        # bytes/s
 
-# HBM bytes per launch of the Winograd GEMM, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# HBM bytes per launch of the Winograd GEMM come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by what the same counters read for a plain copy kernel of known
-# size: x2.0 and x1.0); summary and commands in profiles/gemm_and_transform_40x256_fp16_b64_pmc.txt.
-# Counters cannot be read from inside this process, so the figure is only reported for the
-# workload it was measured on: (blocks, filters, precision, batch).
-MEASURED_GEMM_TRAFFIC = {(40, 256, "fp16", 64): (17792.3 * 2.0 + 28800.0 * 1.0) * 1024.0}
+# size).  Counters cannot be read from inside this process: the figure is read from the
+# tracked summary of those runs, which states it for the workload it was measured on.
+PMC_SUMMARY = os.path.join(ROOT, "profiles", "gemm_and_transform_40x256_fp16_b64_pmc.txt")
+
+
+def measured_gemm_traffic(blocks, filters, precision, batch):
+    """`gemm_traffic_bytes_per_launch = N` of the PMC summary, for its own workload only."""
+    if (blocks, filters, precision, batch) != (40, 256, "fp16", 64):
+        return None
+    try:
+        for line in open(PMC_SUMMARY):
+            if "gemm_traffic_bytes_per_launch" in line and "=" in line:
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def gemm_flops(batch, filters, n_layers):
@@ -190,10 +207,221 @@ def netbench_workload(args, pkg, netgen):
     print(json.dumps(out))
 
 
+def measure_forward(pkg, netgen, torch, blocks, F, precision, B, steps, warmup, lanes_arg,
+                    profile_reps, host_buffers=False, blocks_of_k=0):
+    """One network on the device: evaluations/s of `steps` forwards of B device-resident
+    positions (all lanes, and one lane), optionally the same through host buffers, and the
+    per-kernel-class durations with the roofline figures derived from them."""
+    prec = pkg.FP16 if precision == "fp16" else pkg.FP32
+    net = netgen.make_network(blocks, F, seed=2025)
+    x = netgen.synthetic_inputs(B, seed=2026)
+    w, h = netgen.prepare(net)
+    pipe = pkg.HIPScheduler(prec, B, device=0)
+    pipe.initialize(F)
+    pipe.push_weights(6, 18, F, w)
+    nl = net.n_layers
+
+    d_in = torch.from_numpy(x).cuda()
+    lanes = pipe.lanes() if lanes_arg <= 0 else max(1, min(lanes_arg, pipe.lanes()))
+    d_pols = [torch.zeros(B, 722, device="cuda") for _ in range(lanes)]
+    d_vals = [torch.zeros(B, 361, device="cuda") for _ in range(lanes)]
+    d_pol, d_val = d_pols[0], d_vals[0]
+    torch.cuda.synchronize()
+    ptrs = (d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
+
+    # A step is one forward of one batch.  Steps go to the handle's lanes in turn (a lane is
+    # a stream with the working buffers of one forward), so that `lanes` batches are on the
+    # device side by side, as when the request queue has more callers than one batch holds.
+    def timed(n_lanes, n_steps, n_warm):
+        for i in range(n_warm):
+            k = i % n_lanes
+            pipe.forward_batch_device(B, d_in.data_ptr(), d_pols[k].data_ptr(),
+                                      d_vals[k].data_ptr(), lane=k)
+        pipe.sync()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_steps):
+            k = i % n_lanes
+            pipe.forward_batch_device(B, d_in.data_ptr(), d_pols[k].data_ptr(),
+                                      d_vals[k].data_ptr(), lane=k)
+        pipe.sync()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    dt1 = timed(1, steps, warmup) if lanes > 1 else None
+    dt = timed(lanes, steps, warmup)          # the headline figure: exactly `steps` steps
+    if dt1 is None:
+        dt1 = dt
+    res = {"value": B * steps / dt, "ms_per_step": dt / steps * 1e3, "lanes": lanes,
+           "one_lane": {"value": B * steps / dt1, "unit": "evals/s",
+                        "ms_per_step": dt1 / steps * 1e3,
+                        "note": "the same steps one after the other on one stream: the latency "
+                                "of one batch"}}
+    if blocks_of_k:
+        # the same timed region again, blocks_of_k times: spread of the figure on this box
+        rates = sorted(B * steps / timed(lanes, steps, 2) for _ in range(blocks_of_k))
+        rates1 = sorted(B * steps / timed(1, steps, 2) for _ in range(blocks_of_k))
+        res["blocks_of_k"] = {"blocks": blocks_of_k, "forwards_per_block": steps,
+                              "median": rates[len(rates) // 2], "min": rates[0], "max": rates[-1],
+                              "one_lane_median": rates1[len(rates1) // 2], "unit": "evals/s"}
+
+    if host_buffers:
+        # the same batch handed over as host buffers (pageable numpy arrays in and out): copy
+        # to pinned staging, H2D, forward, D2H, copy out -- PCIe inside the timed region
+        host_steps = max(3, steps // 2)
+        pipe.forward_batch(x)
+        t0 = time.perf_counter()
+        for _ in range(host_steps):
+            pipe.forward_batch(x)
+        host_dt = (time.perf_counter() - t0) / host_steps
+        # ... and from as many threads as the handle has lanes, a batch each at a time
+        host2_dt = None
+        if lanes > 1:
+            import threading
+
+            def host_caller():
+                for _ in range(host_steps):
+                    pipe.forward_batch(x)
+            th = [threading.Thread(target=host_caller) for _ in range(lanes)]
+            t0 = time.perf_counter()
+            for t in th:
+                t.start()
+            for t in th:
+                t.join()
+            host2_dt = (time.perf_counter() - t0) / (host_steps * lanes)
+        res["host_buffers"] = {
+            "value": B / host_dt, "unit": "evals/s", "ms_per_step": host_dt * 1e3,
+            "forwards": host_steps,
+            "note": "lzhip_forward_batch on pageable host arrays, sequential calls: H2D + tower "
+                    "+ 1x1 heads + D2H (PCIe and staging copies inside the timed region)",
+            "callers_as_lanes": (None if host2_dt is None else
+                                 {"value": B / host2_dt, "callers": lanes,
+                                  "note": "one calling thread per lane, a batch each at a time"})}
+
+    # per-kernel-class device time, measured live with HIP events on the pipe's stream
+    ms = np.zeros(pkg.K_COUNT)
+    cnt = np.zeros(pkg.K_COUNT)
+    for _ in range(profile_reps):
+        m, c = pipe.profile_forward(B, *ptrs)
+        ms += m
+        cnt += c
+    ms /= profile_reps
+    cnt /= profile_reps
+    # the same event-timed forward on lane 0 while another lane works through forwards of
+    # its own: what a launch takes when it shares the device, as in the timed steps above
+    ms2 = None
+    if lanes > 1:
+        ms2 = np.zeros(pkg.K_COUNT)
+        for _ in range(profile_reps):
+            for _ in range(3):
+                pipe.forward_batch_device(B, d_in.data_ptr(), d_pols[1].data_ptr(),
+                                          d_vals[1].data_ptr(), lane=1)
+            m, _c = pipe.profile_forward(B, *ptrs)
+            pipe.sync()
+            ms2 += m
+        ms2 /= profile_reps
+    e = 2 if prec == pkg.FP16 else 4
+    gf = gemm_flops(B, F, nl)
+    in_b, out_b, fused_b = transform_bytes(B, F, nl, e)
+    peak = PEAK_MFMA_F16 if prec == pkg.FP16 else PEAK_MFMA_F32
+    gemm_rate = gf / (ms[pkg.K_GEMM] * 1e-3)
+    Fp = (F + 63) // 64 * 64
+    roofline = {
+        "kernel": ("wino_gemm_stream_k" if (prec == pkg.FP16 and Fp == 256) else
+                   "wino_gemm_k / wino_gemm_big_k family") + " (36-way batched Winograd GEMM)",
+        "bound": "mfma", "achieved": gemm_rate / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
+        "frac": gemm_rate / peak,
+        "traffic": measured_gemm_traffic(blocks, F, precision, B),
+        "algorithmic_bytes_per_launch": 36.0 * e * (25 * B * F * 2 + F * F),
+        "avg_launch_us": ms[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],
+        "launches_per_forward": int(cnt[pkg.K_GEMM]),
+        "flops_per_launch": gf / cnt[pkg.K_GEMM],
+    }
+    roofline["launch_context"] = ("launches that run alone (event-timed forward on one lane, "
+                                  "nothing else enqueued)")
+    if ms2 is not None:
+        roofline["side_by_side"] = {
+            "avg_launch_us": ms2[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],
+            "frac": gf / (ms2[pkg.K_GEMM] * 1e-3) / peak,
+            "note": "the same launches while another lane's forward shares the device: each "
+                    "lasts longer, two are in progress"}
+    # the same launch against the HBM roof: at this batch the GEMM's flop-per-byte ratio is below
+    # the machine's (peak flops / peak bytes), so HBM, not MFMA, is the roof above it
+    alg_bytes = roofline["algorithmic_bytes_per_launch"]
+    roofline["flop_per_byte"] = roofline["flops_per_launch"] / alg_bytes
+    roofline["machine_flop_per_byte"] = peak / PEAK_HBM
+    roofline["hbm_view"] = {
+        "achieved": alg_bytes / (roofline["avg_launch_us"] * 1e-6) / 1e9, "peak": PEAK_HBM / 1e9,
+        "unit": "GB/s", "frac": alg_bytes / (roofline["avg_launch_us"] * 1e-6) / PEAK_HBM}
+
+    def hbm(nbytes, k):
+        if cnt[k] == 0:
+            return None
+        rate = nbytes / (ms[k] * 1e-3)
+        return {"bound": "hbm", "achieved": rate / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                "frac": rate / PEAK_HBM, "bytes_per_launch": nbytes / cnt[k],
+                "avg_launch_us": ms[k] * 1e3 / cnt[k], "launches_per_forward": int(cnt[k])}
+
+    res["roofline"] = roofline
+    res["roofline_transforms"] = {"out_in_transform": hbm(fused_b, pkg.K_OUTIN),
+                                  "in_transform": hbm(in_b, pkg.K_IN),
+                                  "out_transform": hbm(out_b, pkg.K_OUT)}
+    res["kernel_ms_per_forward"] = {pkg.KERNEL_CLASSES[k]: float(ms[k]) for k in range(pkg.K_COUNT)}
+    res["_net"], res["_x"], res["_pol"] = net, x, d_pol.cpu().numpy()
+    pipe.close()
+    return res
+
+
+def copy_floor(torch, B, F, e):
+    """What a plain device copy of the GEMM's tile arrays takes on this box: V-sized read +
+    M-sized write (36 x 25B x F elements each) per launch, launches back to back over three
+    buffer pairs, timed with events on the stream they run on."""
+    n = 36 * 25 * B * F
+    dt = torch.float16 if e == 2 else torch.float32
+    src = [torch.ones(n, dtype=dt, device="cuda") for _ in range(3)]
+    dst = [torch.empty(n, dtype=dt, device="cuda") for _ in range(3)]
+    for i in range(6):
+        dst[i % 3].copy_(src[i % 3])
+    torch.cuda.synchronize()
+    reps = 60
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(reps):
+        dst[(i + 1) % 3].copy_(src[i % 3])
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / reps
+    nbytes = 2.0 * n * e
+    return {"us_per_launch": us, "bytes_per_launch": nbytes, "achieved": nbytes / (us * 1e-6) / 1e9,
+            "unit": "GB/s", "frac_of_hbm_peak": nbytes / (us * 1e-6) / PEAK_HBM,
+            "note": "device-to-device copy of a V-sized array into an M-sized one (the bytes a "
+                    "GEMM launch moves, less the filters), launch to launch"}
+
+
+def side_config(pkg, netgen, torch, blocks, F, precision, B, args, cpu=False):
+    """One line for a configuration beside the headline one."""
+    r = measure_forward(pkg, netgen, torch, blocks, F, precision, B, max(20, args.steps // 2),
+                        args.warmup, 0, 2)
+    net, x = r.pop("_net"), r.pop("_x")
+    r.pop("_pol")
+    t = r["roofline_transforms"]["out_in_transform"]
+    out = {"value": r["value"], "unit": "evals/s", "lanes": r["lanes"],
+           "one_lane": r["one_lane"]["value"], "ms_per_batch_one_lane": r["one_lane"]["ms_per_step"],
+           "gemm_frac_of_mfma_peak": r["roofline"]["frac"],
+           "gemm_us_per_launch": r["roofline"]["avg_launch_us"],
+           "transform_frac_of_hbm_peak": t["frac"] if t else None,
+           "transform_us_per_launch": t["avg_launch_us"] if t else None}
+    if cpu and not args.no_cpu_baseline:
+        orc = entry.load_oracle()
+        c, _ = cpu_baseline(orc, netgen, net, x, seconds_budget=3.0)
+        out["cpu_oracle"] = {"value": c["value"], "cores": c["cores"], "sample": c["sample"]}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--blocks", type=int, default=40)
     ap.add_argument("--filters", type=int, default=256)
@@ -201,6 +429,8 @@ def main():
                     help="max batch: default 64 (forward) or 32 (search)")
     ap.add_argument("--precision", choices=["fp16", "fp32"], default="fp16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="forward workload: skip the fp32 run and the smaller configurations")
     ap.add_argument("--profile-reps", type=int, default=5)
     ap.add_argument("--lanes", type=int, default=0,
                     help="forward workload: batches kept on the device side by side; 0 = as "
@@ -252,181 +482,54 @@ def main():
         return
 
     B, F, blocks = args.batch, args.filters, args.blocks
-    prec = pkg.FP16 if args.precision == "fp16" else pkg.FP32
-    net = netgen.make_network(blocks, F, seed=2025)
-    x = netgen.synthetic_inputs(B, seed=2026)
-    w, h = netgen.prepare(net)
-    pipe = pkg.HIPScheduler(prec, B, device=0)
-    pipe.initialize(F)
-    pipe.push_weights(6, 18, F, w)
-    nl = net.n_layers
-
-    d_in = torch.from_numpy(x).cuda()
-    lanes = pipe.lanes() if args.lanes <= 0 else max(1, min(args.lanes, pipe.lanes()))
-    d_pols = [torch.zeros(B, 722, device="cuda") for _ in range(lanes)]
-    d_vals = [torch.zeros(B, 361, device="cuda") for _ in range(lanes)]
-    d_pol, d_val = d_pols[0], d_vals[0]
-    torch.cuda.synchronize()
-    ptrs = (d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
-
-    # A step is one forward of one batch.  Steps go to the handle's lanes in turn (a lane is
-    # a stream with the working buffers of one forward), so that `lanes` batches are on the
-    # device side by side, as when the request queue has more callers than one batch holds.
-    def timed(n_lanes, steps):
-        for i in range(args.warmup):
-            k = i % n_lanes
-            pipe.forward_batch_device(B, d_in.data_ptr(), d_pols[k].data_ptr(),
-                                      d_vals[k].data_ptr(), lane=k)
-        pipe.sync()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            k = i % n_lanes
-            pipe.forward_batch_device(B, d_in.data_ptr(), d_pols[k].data_ptr(),
-                                      d_vals[k].data_ptr(), lane=k)
-        pipe.sync()
-        torch.cuda.synchronize()
-        return time.perf_counter() - t0
-
-    dt1 = timed(1, args.steps) if lanes > 1 else None
-    dt = timed(lanes, args.steps)
-    if dt1 is None:
-        dt1 = dt
-    ms_per_step = dt / args.steps * 1e3
-    evals = B * args.steps / dt
-
-    # the same batch handed over as host buffers (pageable numpy arrays in and out): copy to
-    # pinned staging, H2D, forward, D2H, copy out, one batch at a time -- reported beside the
-    # headline figure, never as it
-    host_steps = max(3, args.steps // 2)
-    pipe.forward_batch(x)
-    t0 = time.perf_counter()
-    for _ in range(host_steps):
-        pipe.forward_batch(x)
-    host_dt = (time.perf_counter() - t0) / host_steps
-    # ... and from as many threads as the handle has lanes, a batch each at a time
-    host2_dt = None
-    if lanes > 1:
-        import threading
-
-        def host_caller():
-            for _ in range(host_steps):
-                pipe.forward_batch(x)
-        th = [threading.Thread(target=host_caller) for _ in range(lanes)]
-        t0 = time.perf_counter()
-        for t in th:
-            t.start()
-        for t in th:
-            t.join()
-        host2_dt = (time.perf_counter() - t0) / (host_steps * lanes)
-
-    # per-kernel-class device time, measured live with HIP events on the pipe's stream
-    ms = np.zeros(pkg.K_COUNT)
-    cnt = np.zeros(pkg.K_COUNT)
-    for _ in range(args.profile_reps):
-        m, c = pipe.profile_forward(B, *ptrs)
-        ms += m
-        cnt += c
-    ms /= args.profile_reps
-    cnt /= args.profile_reps
-    # the same event-timed forward on lane 0 while another lane works through forwards of
-    # its own: what a launch takes when it shares the device, as in the timed steps above
-    ms2 = None
-    if lanes > 1:
-        ms2 = np.zeros(pkg.K_COUNT)
-        for _ in range(args.profile_reps):
-            for _ in range(3):
-                pipe.forward_batch_device(B, d_in.data_ptr(), d_pols[1].data_ptr(),
-                                          d_vals[1].data_ptr(), lane=1)
-            m, _c = pipe.profile_forward(B, *ptrs)
-            pipe.sync()
-            ms2 += m
-        ms2 /= args.profile_reps
-    e = 2 if prec == pkg.FP16 else 4
-    gf = gemm_flops(B, F, nl)
-    in_b, out_b, fused_b = transform_bytes(B, F, nl, e)
-    peak = PEAK_MFMA_F16 if prec == pkg.FP16 else PEAK_MFMA_F32
-    gemm_rate = gf / (ms[pkg.K_GEMM] * 1e-3)
-    roofline = {
-        "kernel": "wino_gemm_split_k / wino_gemm_k family (36-way batched Winograd GEMM)",
-        "bound": "mfma", "achieved": gemm_rate / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
-        "frac": gemm_rate / peak,
-        "traffic": MEASURED_GEMM_TRAFFIC.get((blocks, F, args.precision, B)),
-        "algorithmic_bytes_per_launch": 36.0 * e * (25 * B * F * 2 + F * F),
-        "avg_launch_us": ms[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],
-        "launches_per_forward": int(cnt[pkg.K_GEMM]),
-        "flops_per_launch": gf / cnt[pkg.K_GEMM],
-    }
-    roofline["launch_context"] = ("launches that run alone (event-timed forward on one lane, "
-                                  "nothing else enqueued)")
-    if ms2 is not None:
-        roofline["side_by_side"] = {
-            "avg_launch_us": ms2[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],
-            "frac": gf / (ms2[pkg.K_GEMM] * 1e-3) / peak,
-            "note": "the same launches while another lane's forward shares the device: each "
-                    "lasts longer, two are in progress"}
-    # the same launch against the HBM roof: at this batch the GEMM's flop-per-byte ratio is below
-    # the machine's (peak flops / peak bytes), so HBM, not MFMA, is the roof above it
-    alg_bytes = roofline["algorithmic_bytes_per_launch"]
-    roofline["flop_per_byte"] = roofline["flops_per_launch"] / alg_bytes
-    roofline["machine_flop_per_byte"] = peak / PEAK_HBM
-    roofline["hbm_view"] = {
-        "achieved": alg_bytes / (roofline["avg_launch_us"] * 1e-6) / 1e9, "peak": PEAK_HBM / 1e9,
-        "unit": "GB/s", "frac": alg_bytes / (roofline["avg_launch_us"] * 1e-6) / PEAK_HBM}
-
-    def hbm(nbytes, k):
-        if cnt[k] == 0:
-            return None
-        rate = nbytes / (ms[k] * 1e-3)
-        return {"bound": "hbm", "achieved": rate / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s",
-                "frac": rate / PEAK_HBM, "bytes_per_launch": nbytes / cnt[k],
-                "avg_launch_us": ms[k] * 1e3 / cnt[k], "launches_per_forward": int(cnt[k])}
-
-    transforms = {"out_in_transform": hbm(fused_b, pkg.K_OUTIN),
-                  "in_transform": hbm(in_b, pkg.K_IN),
-                  "out_transform": hbm(out_b, pkg.K_OUT)}
-    kernel_ms = {pkg.KERNEL_CLASSES[k]: float(ms[k]) for k in range(pkg.K_COUNT)}
+    head = measure_forward(pkg, netgen, torch, blocks, F, args.precision, B, args.steps,
+                           args.warmup, args.lanes, args.profile_reps, host_buffers=True,
+                           blocks_of_k=5)
+    net, x = head.pop("_net"), head.pop("_x")
+    pol = head.pop("_pol")
 
     # parity spot check + CPU baseline (oracle as checker / reported baseline only)
     cpu = None
     if not args.no_cpu_baseline:
         orc = entry.load_oracle()
         cpu, (rpol, rval) = cpu_baseline(orc, netgen, net, x)
-        pol = d_pol.cpu().numpy()
         k = min(B, rpol.shape[0])
         rel = float(np.linalg.norm(pol[:k] - rpol[:k]) / max(np.linalg.norm(rpol[:k]), 1e-30))
         cpu["raw_policy_plane_rel_l2_vs_gpu"] = rel
-    pipe.close()
 
     out = {
         "metric": "NN evals/sec at 40x256 fp16 b64 on 1 MI355X; Winograd GEMM MFMA util %",
-        "value": evals, "unit": "evals/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "value": head["value"], "unit": "evals/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 storage, f32 accumulate" if prec == pkg.FP16 else "f32",
+        "dtype": "f16 storage, f32 accumulate" if args.precision == "fp16" else "f32",
         "data": "synthetic",
         "config": {"workload": "%d blocks x %d filters, %s, batch %d (the headline configuration when "
                                "40x256 fp16 b64), %d conv layers + 1x1 heads per step"
-                               % (blocks, F, args.precision, B, nl),
+                               % (blocks, F, args.precision, B, net.n_layers),
                    "inputs": "device-resident fp32 NCHW [%d][18][361]" % B,
-                   "lanes": lanes},
-        "one_lane": {"value": B * args.steps / dt1, "unit": "evals/s",
-                     "ms_per_step": dt1 / args.steps * 1e3,
-                     "note": "the same steps one after the other on one stream: the latency "
-                             "of one batch"},
-        "roofline": roofline,
-        "roofline_transforms": transforms,
-        "kernel_ms_per_forward": kernel_ms,
-        "gemm_mfma_util_pct": 100.0 * gemm_rate / peak,
-        "host_buffers": {"value": B / host_dt, "unit": "evals/s", "ms_per_step": host_dt * 1e3,
-                         "note": "lzhip_forward_batch on pageable host arrays, sequential calls "
-                                 "(PCIe and staging copies inside the timed region)",
-                         "callers_as_lanes": (None if host2_dt is None else
-                                              {"value": B / host2_dt, "callers": lanes})},
+                   "lanes": head["lanes"]},
+        "blocks_of_k": head["blocks_of_k"],
+        "one_lane": head["one_lane"],
+        "host_buffers": head["host_buffers"],
+        "roofline": head["roofline"],
+        "roofline_transforms": head["roofline_transforms"],
+        "kernel_ms_per_forward": head["kernel_ms_per_forward"],
+        "gemm_mfma_util_pct": 100.0 * head["roofline"]["frac"],
+        "hbm_copy_floor": copy_floor(torch, B, F, 2 if args.precision == "fp16" else 4),
         "cpu_baseline": cpu,
-        "environment": {"device": torch.cuda.get_device_name(0), "hip": torch.version.hip,
-                        "torch": torch.__version__},
     }
+    if not args.headline_only:
+        # the same network in fp32, and the three smaller configurations, one line each
+        if args.precision == "fp16":
+            out["fp32"] = side_config(pkg, netgen, torch, blocks, F, "fp32", B, args)
+        out["configs"] = {
+            "6x128 fp32 b1": side_config(pkg, netgen, torch, 6, 128, "fp32", 1, args, cpu=True),
+            "15x192 fp32 b8": side_config(pkg, netgen, torch, 15, 192, "fp32", 8, args),
+            "20x256 fp16 b32": side_config(pkg, netgen, torch, 20, 256, "fp16", 32, args),
+        }
+    out["environment"] = {"device": torch.cuda.get_device_name(0), "hip": torch.version.hip,
+                          "torch": torch.__version__}
     print(json.dumps(out))
 
 

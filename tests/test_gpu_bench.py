@@ -46,6 +46,19 @@ def test_forward_line():
     for name in ("out_in_transform", "in_transform", "out_transform"):
         t = d["roofline_transforms"][name]
         assert t["bound"] == "hbm" and 0 < t["frac"] < 1
+    # the figures beside the headline one: host buffers (PCIe inside the timed region), the
+    # repeated blocks, the plain-copy floor, the same net in fp32 and the smaller configurations
+    hb = d["host_buffers"]
+    assert hb["value"] > 0 and "PCIe" in hb["note"] and d["config"]["inputs"].startswith("device")
+    bk = d["blocks_of_k"]
+    assert bk["blocks"] == 5 and bk["forwards_per_block"] == 3 and bk["min"] <= bk["median"] <= bk["max"]
+    cf = d["hbm_copy_floor"]
+    assert cf["us_per_launch"] > 0 and 0 < cf["frac_of_hbm_peak"] < 1.5
+    assert d["fp32"]["value"] > 0 and 0 < d["fp32"]["gemm_frac_of_mfma_peak"] < 1
+    assert set(d["configs"]) == {"6x128 fp32 b1", "15x192 fp32 b8", "20x256 fp16 b32"}
+    for c in d["configs"].values():
+        assert c["value"] > 0 and c["one_lane"] > 0
+    assert d["configs"]["6x128 fp32 b1"]["cpu_oracle"]["value"] > 0
 
 
 def test_more_than_one_gpu_is_refused():
