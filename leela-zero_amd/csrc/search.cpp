@@ -276,15 +276,42 @@ struct Node {
     }
     // Mean value for `tomove` with `vl` pending visits counted as losses.
     float raw_eval(int tomove, int vl) const {
-        const int v = visits.load() + vl;
-        double be = blackevals.load();
-        if (tomove == go::WHITE) be += (double)vl;
-        float e = v > 0 ? (float)(be / (double)v) : 0.5f;
-        if (tomove == go::WHITE) e = 1.0f - e;
-        return e;
+        return puct_eval_for(tomove, blackevals.load(), visits.load(), vl);
     }
     bool expanded() const { return state.load(std::memory_order_acquire) == ST_EXPANDED; }
 };
+
+float puct_eval_for(int tomove, double blackevals, int visits, int virtual_loss) {
+    const int v = visits + virtual_loss;
+    double be = blackevals;
+    if (tomove == go::WHITE) be += (double)virtual_loss;
+    float e = v > 0 ? (float)(be / (double)v) : 0.5f;
+    if (tomove == go::WHITE) e = 1.0f - e;
+    return e;
+}
+
+PuctParent puct_parent(const lzhip_search_config& cfg, size_t children_visits,
+                       float visited_policy, float parent_eval_for_color) {
+    PuctParent p;
+    p.numerator = std::sqrt((double)children_visits *
+                            std::log((double)cfg.logpuct * (double)children_visits +
+                                     (double)cfg.logconst));
+    p.fpu_reduction = cfg.fpu_reduction * std::sqrt(visited_policy);
+    p.fpu_eval = parent_eval_for_color - p.fpu_reduction;
+    return p;
+}
+
+double puct_value(const lzhip_search_config& cfg, const PuctParent& parent, float prior,
+                  int visits, bool expanding, float child_eval_for_color) {
+    float winrate = parent.fpu_eval;
+    if (expanding)
+        winrate = -1.0f - parent.fpu_reduction;  // someone is waiting for its evaluation
+    else if (visits > 0)
+        winrate = child_eval_for_color;
+    const double puct =
+        (double)cfg.puct * (double)prior * (parent.numerator / (1.0 + (double)visits));
+    return (double)winrate + puct;
+}
 
 static void free_tree(Node* n) {
     if (!n) return;
@@ -448,10 +475,8 @@ Child* UCTSearch::select_child(Node* node, int color, bool /*is_root*/) {
         parentvisits += (size_t)v;
         if (v > 0) total_visited_policy += c.prior;
     }
-    const double numerator = std::sqrt(
-        (double)parentvisits * std::log((double)m_cfg.logpuct * (double)parentvisits + (double)m_cfg.logconst));
-    const float fpu_reduction = m_cfg.fpu_reduction * std::sqrt(total_visited_policy);
-    const float fpu_eval = node->raw_eval(color, 0) - fpu_reduction;
+    const PuctParent parent =
+        puct_parent(m_cfg, parentvisits, total_visited_policy, node->raw_eval(color, 0));
 
     Child* best = nullptr;
     double best_value = std::numeric_limits<double>::lowest();
@@ -460,14 +485,11 @@ Child* UCTSearch::select_child(Node* node, int color, bool /*is_root*/) {
         if (!c.valid.load(std::memory_order_relaxed)) continue;
         Node* n = c.node.load(std::memory_order_acquire);
         const int v = n ? n->visits.load(std::memory_order_relaxed) : 0;
-        float winrate = fpu_eval;
-        if (n && n->state.load(std::memory_order_relaxed) == ST_EXPANDING) {
-            winrate = -1.0f - fpu_reduction;  // someone is waiting for its evaluation
-        } else if (v > 0) {
-            winrate = n->raw_eval(color, n->vloss.load(std::memory_order_relaxed));
-        }
-        const double puct = (double)m_cfg.puct * (double)c.prior * (numerator / (1.0 + (double)v));
-        const double value = (double)winrate + puct;
+        const bool expanding = n && n->state.load(std::memory_order_relaxed) == ST_EXPANDING;
+        const float child_eval =
+            (v > 0 && !expanding) ? n->raw_eval(color, n->vloss.load(std::memory_order_relaxed))
+                                  : 0.0f;
+        const double value = puct_value(m_cfg, parent, c.prior, v, expanding, child_eval);
         if (value > best_value) {
             best_value = value;
             best = &c;

@@ -143,6 +143,29 @@ struct SearchStats {
 struct Node;
 struct Child;
 
+// The arithmetic of child selection on plain numbers, as UCTNode::uct_select_child and
+// UCTNode::get_raw_eval do it (reference src/UCTNode.cpp:306-362, :270-282); the tree code
+// below calls exactly these, and the host tests pin them on hand-worked nodes.
+//
+// Mean value of a node for `tomove` with `virtual_loss` visits in progress counted as
+// lost: blackevals / (visits + vl) for black; for white the pending visits count as black
+// wins before the value is turned round.  0.5 for a node without visits.
+float puct_eval_for(int tomove, double blackevals, int visits, int virtual_loss);
+// What the parent contributes: the exploration numerator sqrt(N ln(logpuct N + logconst))
+// over the children's visits N, and the value given to children without visits, the
+// parent's own mean for the side to move less fpu_reduction * sqrt(priors of the visited).
+struct PuctParent {
+    double numerator;
+    float fpu_reduction;
+    float fpu_eval;
+};
+PuctParent puct_parent(const lzhip_search_config& cfg, size_t children_visits,
+                       float visited_policy, float parent_eval_for_color);
+// Selection value of one child: its mean (fpu_eval without visits, -1 - fpu_reduction
+// while another thread expands it) + puct * prior * numerator / (1 + visits).
+double puct_value(const lzhip_search_config& cfg, const PuctParent& parent, float prior,
+                  int visits, bool expanding, float child_eval_for_color);
+
 class UCTSearch {
 public:
     UCTSearch(NetworkFacade& net, const lzhip_search_config& cfg);

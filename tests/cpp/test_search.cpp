@@ -417,7 +417,85 @@ static void test_selfplay_entry_and_failure() {
     }
 }
 
+// Child selection on a hand-worked node (reference src/UCTNode.cpp:306-362, get_raw_eval
+// :270-282, defaults src/GTP.cpp:346-350: puct 0.5, logpuct 0.015, logconst 1.7, fpu
+// reduction 0.25; virtual loss 3, src/UCTNode.h:51).
+//
+// Parent: mean for black 0.55.  Children (prior, visits, sum of black values):
+//   c0 0.40, 6, 3.30      c1 0.30, 3, 1.95      c2 0.20, 0      c3 0.10, 0
+// N = 9 visits below the parent, priors of the visited children 0.70.
+//   numerator     = sqrt(9 * ln(0.015 * 9 + 1.7)) = sqrt(9 * 0.607045) = 2.337392
+//   fpu_reduction = 0.25 * sqrt(0.70) = 0.209165
+// Black to move: fpu_eval = 0.55 - 0.209165 = 0.340835
+//   c0  3.30/6 = 0.55   + 0.5 * 0.40 * 2.337392 / 7 = 0.55 + 0.066783 = 0.616783
+//   c1  1.95/3 = 0.65   + 0.5 * 0.30 * 2.337392 / 4 = 0.65 + 0.087652 = 0.737652   <- chosen
+//   c2  0.340835        + 0.5 * 0.20 * 2.337392 / 1 =                   0.574574
+//   c3  0.340835        + 0.5 * 0.10 * 2.337392 / 1 =                   0.457705
+//   Without the reduction c2 would read 0.55 + 0.233739 = 0.783739 and be chosen (and with
+//   the reduction added instead of subtracted, 0.992904): the reduction decides.
+// White to move: parent mean 0.45, fpu_eval = 0.240835; the children's means turn round
+//   c0  0.45 + 0.066783 = 0.516783   <- chosen     c1  0.35 + 0.087652 = 0.437652
+//   c2  0.240835 + 0.233739 = 0.474574             c3  0.240835 + 0.116870 = 0.357705
+// Virtual loss, black to move, another thread inside c1 (3 pending visits counted as lost):
+//   c1  1.95/(3+3) = 0.325 + 0.087652 = 0.412652, so c0 (0.616783) is chosen instead;
+//   seen from white the three pending visits count as black wins: 1 - (1.95+3)/6 = 0.175.
+// A child under expansion reads -1 - 0.209165 + its exploration term and is never chosen
+// while another child is there.
+static void test_puct_arithmetic() {
+    lzhip_search_config cfg = config(1, 10, 1);
+    CHECK(cfg.puct == 0.5f && cfg.logpuct == 0.015f && cfg.logconst == 1.7f);
+    CHECK(cfg.fpu_reduction == 0.25f && cfg.virtual_loss == 3);
+    const float prior[4] = {0.40f, 0.30f, 0.20f, 0.10f};
+    const int visits[4] = {6, 3, 0, 0};
+    const double blackevals[4] = {3.30, 1.95, 0.0, 0.0};
+    auto near = [](double a, double b) { return std::fabs(a - b) < 2e-6; };
+    auto pick = [&](const lzhip_search_config& c, int color, const int* vloss, int expanding,
+                    double* values) {
+        size_t n = 0;
+        float visited = 0.0f;
+        for (int i = 0; i < 4; i++) {
+            n += (size_t)visits[i];
+            if (visits[i] > 0) visited += prior[i];
+        }
+        const float parent_eval = puct_eval_for(color, 5.5, 10, 0);
+        const PuctParent par = puct_parent(c, n, visited, parent_eval);
+        int best = -1;
+        double best_value = -1e300;
+        for (int i = 0; i < 4; i++) {
+            const float e = puct_eval_for(color, blackevals[i], visits[i], vloss ? vloss[i] : 0);
+            values[i] = puct_value(c, par, prior[i], visits[i], i == expanding, e);
+            if (values[i] > best_value) {
+                best_value = values[i];
+                best = i;
+            }
+        }
+        return best;
+    };
+    double v[4];
+    {
+        const PuctParent par = puct_parent(cfg, 9, 0.70f, 0.55f);
+        CHECK(near(par.numerator, 2.337392) && near(par.fpu_reduction, 0.209165) &&
+              near(par.fpu_eval, 0.340835));
+    }
+    CHECK(pick(cfg, go::BLACK, nullptr, -1, v) == 1);
+    CHECK(near(v[0], 0.616783) && near(v[1], 0.737652) && near(v[2], 0.574574) &&
+          near(v[3], 0.457705));
+    lzhip_search_config no_fpu = cfg;
+    no_fpu.fpu_reduction = 0.0f;
+    CHECK(pick(no_fpu, go::BLACK, nullptr, -1, v) == 2 && near(v[2], 0.783739));
+    CHECK(pick(cfg, go::WHITE, nullptr, -1, v) == 0);
+    CHECK(near(v[0], 0.516783) && near(v[1], 0.437652) && near(v[2], 0.474574) &&
+          near(v[3], 0.357705));
+    const int vloss[4] = {0, 3, 0, 0};
+    CHECK(pick(cfg, go::BLACK, vloss, -1, v) == 0 && near(v[1], 0.412652));
+    CHECK(near(puct_eval_for(go::WHITE, 1.95, 3, 3), 0.175));
+    CHECK(near(puct_eval_for(go::BLACK, 0.0, 0, 0), 0.5));
+    CHECK(pick(cfg, go::BLACK, nullptr, 1, v) == 0 && near(v[1], -1.0 - 0.209165 + 0.087652));
+    std::printf("puct arithmetic pinned\n");
+}
+
 int main() {
+    test_puct_arithmetic();
     std::printf("unrotation\n");
     test_unrotation();
     test_value_head_not_stm();
