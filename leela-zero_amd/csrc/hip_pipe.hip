@@ -781,7 +781,7 @@ private:
                                             m_Fp, m_Tp, ln.stream, nullptr);
                 }
                 const float mx = absmax(dst, cnt);
-                if (!(mx < 60000.0f)) {  // saturated (or NaN): coarser scale, try again
+                if (!(mx < kActStoreMax)) {  // at the storage clamp (or NaN): coarser scale, try again
                     m_s[l + 1] *= 256.0f;
                     adjusted = false;
                     continue;

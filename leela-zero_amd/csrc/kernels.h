@@ -22,6 +22,9 @@ constexpr int kPos = 36;       // 6x6 Winograd positions
 constexpr int kInPlanes = 18;
 constexpr int kGemmBM = 128;   // row extent of the standard GEMM tile
 constexpr int kTileRowPad = 256;  // V and M row counts (Tp) are multiples of this
+// Largest magnitude an activation is stored with in half precision (see act_clamp in
+// kernels.hip); the calibration treats a measured maximum at this value as saturated.
+constexpr float kActStoreMax = 2040.0f;
 
 // Timing hook: when non-null every launch is bracketed by this event pair
 // (device begin/end timestamps of that launch alone).

@@ -58,6 +58,20 @@ template <> __device__ __forceinline__ half_t to_storage<half_t>(float v) {
     return (half_t)fminf(fmaxf(v, -65504.0f), 65504.0f);
 }
 
+// Stored activations are kept at or below kActStoreMax = 2040 < 65504 / 30.6 (30.6 = largest
+// absolute row sum of B^T (x) B^T), so the input transform of a stored activation cannot
+// leave the half-precision range and V needs no clamp of its own.  Every kernel that
+// stores an activation (fused and unfused output transform) goes through this one clamp,
+// and the activation-scale calibration measures through it.
+template <typename P> __device__ __forceinline__ float act_clamp(float v);
+template <> __device__ __forceinline__ float act_clamp<float>(float v) { return v; }
+template <> __device__ __forceinline__ float act_clamp<half_t>(float v) {
+    return fminf(v, kActStoreMax);
+}
+template <typename P> __device__ __forceinline__ P act_to_storage(float v) {
+    return (P)act_clamp<P>(v);
+}
+
 // o = B^T i for one 6-vector (reference src/CPUPipe.cpp:88-106).
 __device__ __forceinline__ void bt6(const float i0, const float i1, const float i2,
                                     const float i3, const float i4, const float i5, float& o0,
@@ -302,7 +316,8 @@ __global__ __launch_bounds__(256) void out_transform_k(
             float val[VN];
 #pragma unroll
             for (int v = 0; v < VN; v++)
-                val[v] = fmaxf(0.0f, sc[v] * (o[v][i * 4 + jj] - mn[v]) + rfac * r[v][i * 4 + jj]);
+                val[v] = act_clamp<P>(
+                    fmaxf(0.0f, sc[v] * (o[v][i * 4 + jj] - mn[v]) + rfac * r[v][i * 4 + jj]));
             if (y < kBoard && x < kBoard)
                 ChanVec<P>::store(out + bbase + (size_t)(y * kBoard + x) * Kp, val);
         }
@@ -408,15 +423,6 @@ template <typename P>
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const P* base, size_t bytes) {
     // untyped 32-bit-element descriptor for gfx9-family raw buffer instructions
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<P*>(base), 0, (int)bytes, 0x00020000);
-}
-
-// Stored activations are kept below 65504 / 30.6 (30.6 = largest absolute row
-// sum of B^T (x) B^T), so the input transform of a stored activation cannot
-// leave the half-precision range and V needs no clamp of its own.
-template <typename P> __device__ __forceinline__ P act_to_storage(float v);
-template <> __device__ __forceinline__ float act_to_storage<float>(float v) { return v; }
-template <> __device__ __forceinline__ half_t act_to_storage<half_t>(float v) {
-    return (half_t)fminf(v, 2040.0f);
 }
 
 // One workgroup owns one board and 64 channels.  A lane owns two consecutive

@@ -545,3 +545,42 @@ def test_bit_packed_and_float_requests_agree(pkg, netgen, orc):
         pe, ve = pipe.forward_eval(x[i])
         assert np.abs(pe - policy[i]).max() <= 1e-6 and abs(ve - value[i]) <= 1e-6, i
     pipe.close()
+
+
+def test_fp16_range_beyond_the_calibration_positions(pkg, netgen, orc):
+    """Stored activations are scaled at push_weights from 8 synthetic positions (target
+    maximum 16) and clamped at 2040 on storage, by the fused and the unfused output
+    transform alike.  Planes 64 times larger than anything the calibration saw still sit
+    inside that range and agree with the oracle; planes 4096 times larger run into the clamp
+    and must come out finite, with a policy that sums to one; and a single layer whose
+    outputs exceed the clamp stores exactly min(y, 2040)."""
+    print("case: fp16 range", flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 128, 6100, pkg.FP16, 4)
+    x = netgen.synthetic_inputs(4, seed=61)
+    big = (64.0 * x).astype(np.float32)
+    policy, value, logits, pol, val = pipe.evaluate_batch(big, want_raw=True)
+    for i in range(4):
+        rp, rv = ref.forward(big[i])
+        assert rel_l2(pol[i], rp) <= 2e-2 and rel_l2(val[i], rv) <= 2e-2, i
+    huge = (4096.0 * x).astype(np.float32)
+    policy, value, logits, pol, val = pipe.evaluate_batch(huge, want_raw=True)
+    assert np.isfinite(pol).all() and np.isfinite(val).all() and np.isfinite(logits).all()
+    assert np.isfinite(policy).all() and np.isfinite(value).all()
+    assert np.allclose(policy.sum(axis=1), 1.0, atol=1e-3)
+    # one layer through the unfused kernel, inputs chosen so that many outputs pass 2040
+    rng = np.random.default_rng(62)
+    # (inputs stay inside the stored range themselves, so that V = B^T d B stays in half range)
+    a = np.minimum(np.abs(rng.standard_normal((2, 128, 361))) * 600.0, 2000.0)
+    a = a.astype(np.float16).astype(np.float32)
+    V, M, Y = pipe.debug_layer(1, a)
+    clipped = 0
+    for i in range(2):
+        Vr = orc.transform_in(a[i], 128)
+        Mr = orc.sgemm(ref.U[1], Vr, 128, 128)
+        Yr = orc.batchnorm(orc.transform_out(Mr, 128), ref.mean[1], ref.scale[1])
+        want = np.minimum(Yr, 2040.0)
+        clipped += int((Yr > 2040.0).sum())
+        assert Y[i].max() <= 2040.0
+        assert rel_l2(Y[i], want) <= 4e-3
+    assert clipped > 100, clipped
+    pipe.close()

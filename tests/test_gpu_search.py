@@ -265,3 +265,43 @@ def test_value_head_of_format_2_networks(pkg, netgen, orc, tmp_path):
     assert pipe.get_output(h, boards, b.to_move, 5)[1] == w0
     pipe.close()
 
+
+
+def test_search_configuration_four_at_full_size(pkg, netgen):
+    """BASELINE configs[4] as written: 16 search threads, max batch 32, the 40x256 fp16
+    network, 1600 visits per move, 20 moves from the empty board (the call pattern of the
+    reference's UCTSearch::think, src/UCTSearch.cpp:757-850, threads/batch defaults
+    src/Leela.cpp:64-133).  The fully connected head weights are rescaled as bench.py does
+    it (a deep random-init tower saturates softmax and tanh, and the search would follow a
+    single line); the tower, i.e. the device work per evaluation, is untouched."""
+    import bench
+    print("case: search configs[4] 40x256 fp16, 16 threads, max batch 32", flush=True)
+    net = netgen.make_network(40, 256, seed=2025)
+    w, h = netgen.prepare(net)
+    pipe = pkg.HIPScheduler(pkg.FP16, 32)
+    pipe.initialize(256)
+    pipe.push_weights(6, 18, 256, w)
+    h = bench.calibrate_heads(pipe, netgen, h, 32)
+    pipe.selfplay(h, pkg.SearchConfig.default(threads=16, visits=200, moves=1, seed=1))
+    pipe.reset_stats()
+    cfg = pkg.SearchConfig.default(threads=16, visits=1600, moves=20, seed=2027)
+    res, moves = pipe.selfplay(h, cfg)
+    assert res.moves_played == len(moves) == 20
+    b = G.Board()
+    for mv in moves:
+        assert b.is_legal(b.to_move, mv), mv
+        b.play(mv)
+        assert not (mv != G.PASS and b.superko())
+    assert res.playouts >= 20 * 1000
+    assert res.evals + res.cache_hits == res.cache_lookups
+    assert res.sched.requests + res.sched.halted == res.evals
+    fill = res.sched.requests / res.sched.batch_slots
+    assert res.sched.max_batch_seen <= 32
+    assert 0.45 <= fill <= 0.55, fill       # 16 callers can fill half of 32 at most
+    print("configs[4]: %.0f visits/s, fill %.3f, mean batch %.1f, max batch %d, evals %d, "
+          "halted %d, %.2f s" % (res.visits_per_s, fill,
+                                 res.sched.requests / max(1, res.sched.batches),
+                                 res.sched.max_batch_seen, res.evals, res.halted, res.seconds),
+          flush=True)
+    assert res.visits_per_s > 4000
+    pipe.close()
