@@ -129,6 +129,10 @@ public:
         // Small batches leave more of the device idle at every kernel boundary: a third
         // lane pays up to batch 32 (+10 %) and no longer at 64 (-2 %).
         m_n_lanes = max_batch <= 32 ? 3 : 2;
+        if (const char* e = std::getenv("LZHIP_LANES")) {   // measurement knob: 1..3 lanes
+            const int v = std::atoi(e);
+            if (v >= 1 && v <= kLanes) m_n_lanes = v;
+        }
         // Every refusal comes before the first stream, event or allocation is made: a
         // constructor that throws runs no destructor.
         m_Fp = round_up(filters, 64);
