@@ -409,7 +409,7 @@ public:
                 HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
                               m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
                 launch_heads(sl->dpol.p, sl->dval.p, hp, temperature, sl->hpol.p, nullptr,
-                             sl->hval.p, n, ln.stream);
+                             sl->hval.p, sl->dwork.p, n, ln.stream);
             }
             HIP_CHECK(hipGetLastError());
             HIP_CHECK(hipEventRecord(sl->done, ln.stream));
@@ -430,14 +430,12 @@ public:
         };
         up(m_h[0], hw.bn_pol_mean, 2);
         up(m_h[1], hw.bn_pol_scale, 2);
-        {   // FC matrices go up input-major (what heads_k reads)
-            std::vector<float> t((size_t)722 * 362);
-            for (int o = 0; o < 362; o++)
-                for (int i = 0; i < 722; i++) t[(size_t)i * 362 + o] = hw.ip_pol_w[(size_t)o * 722 + i];
+        {   // FC matrices go up in the operand order of the matrix instruction
+            std::vector<float> t(head_fc_fragment_count(true));
+            head_fc_fragments(hw.ip_pol_w, true, t.data());
             up(m_h[2], t.data(), t.size());
-            t.assign((size_t)361 * 256, 0.0f);
-            for (int o = 0; o < 256; o++)
-                for (int i = 0; i < 361; i++) t[(size_t)i * 256 + o] = hw.ip1_val_w[(size_t)o * 361 + i];
+            t.assign(head_fc_fragment_count(false), 0.0f);
+            head_fc_fragments(hw.ip1_val_w, false, t.data());
             up(m_h[6], t.data(), t.size());
         }
         up(m_h[3], hw.ip_pol_b, 362);
@@ -450,6 +448,8 @@ public:
         m_dpolicy.alloc(B * 362);
         m_dlogits.alloc(B * 362);
         m_dvalue.alloc(B);
+        m_dwork.alloc(B * (362 + 256));
+        for (int i = 0; i < m_n_lanes; i++) m_slot[i].dwork.alloc(B * (362 + 256));
         m_heads_ready = true;
     }
 
@@ -467,7 +467,7 @@ public:
         HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
                       m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
         launch_heads(m_dpol.p, m_dval.p, hp, temperature, m_dpolicy.p, m_dlogits.p, m_dvalue.p,
-                     n, ln.stream);
+                     m_dwork.p, n, ln.stream);
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipStreamSynchronize(ln.stream));
         HIP_CHECK(hipMemcpy(policy, m_dpolicy.p, sizeof(float) * (size_t)n * 362, hipMemcpyDeviceToHost));
@@ -821,6 +821,7 @@ private:
         PinnedBuf<float> hin, hpol, hval;
         PinnedBuf<uint32_t> hbits;
         DevBuf<float> din, dpol, dval;
+        DevBuf<float> dwork;   // heads: logits and hidden units between the two kernels
         hipEvent_t done = nullptr;
         bool busy = false;
     };
@@ -830,7 +831,7 @@ private:
     std::condition_variable m_slot_cv;
     std::vector<Layer> m_layers;
     std::vector<float> m_s;  // activation scales, m_s[0] = input
-    DevBuf<float> m_h[10], m_dpolicy, m_dlogits, m_dvalue;
+    DevBuf<float> m_h[10], m_dpolicy, m_dlogits, m_dvalue, m_dwork;
     bool m_heads_ready = false;
     hipEvent_t m_ev_start[kTimerPool] = {}, m_ev_stop[kTimerPool] = {};
     int m_timer_class[kTimerPool] = {};

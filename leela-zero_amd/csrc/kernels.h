@@ -86,14 +86,21 @@ void launch_head_conv(const P* act, const float* w3, float out_scale, float* pol
 template <typename P>
 void launch_absmax(const P* x, size_t count, float* out, hipStream_t s);
 
-// Head arithmetic above the pipe boundary, one workgroup per position.
-// Device pointers; the two large FC matrices are held input-major:
-// ip_pol_wt [722][362], ip1_val_wt [361][256].
+// Head arithmetic above the pipe boundary: BN + ReLU, the two large fully connected layers
+// on the matrix cores, softmax / FC + tanh.  Device pointers; the two large FC matrices are
+// held in the operand order of the matrix instruction (head_fc_fragments).
 struct HeadParams {
-    const float *bn_pol_mean, *bn_pol_scale, *ip_pol_wt, *ip_pol_b;
-    const float *bn_val_mean, *bn_val_scale, *ip1_val_wt, *ip1_val_b, *ip2_val_w, *ip2_val_b;
+    const float *bn_pol_mean, *bn_pol_scale, *ip_pol_wf, *ip_pol_b;
+    const float *bn_val_mean, *bn_val_scale, *ip1_val_wf, *ip1_val_b, *ip2_val_w, *ip2_val_b;
 };
+// Element count of the fragment-order copy of the policy (true) / value (false) matrix, and
+// its construction from W [outputs][inputs] row-major.
+size_t head_fc_fragment_count(bool policy);
+void head_fc_fragments(const float* W, bool policy, float* dst);
+// work: device scratch of n * (362 + 256) floats (logits and hidden units between the two
+// kernels).  logits may be null.
 void launch_heads(const float* pol, const float* val, HeadParams hp, float temperature,
-                  float* policy, float* logits, float* value, int n, hipStream_t s);
+                  float* policy, float* logits, float* value, float* work, int n,
+                  hipStream_t s);
 
 }  // namespace lzhip

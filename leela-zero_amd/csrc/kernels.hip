@@ -1494,7 +1494,13 @@ __global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restri
             if (lval[i]) *reinterpret_cast<int4v*>(&S[lrow[i] * ROWE + lcc[i] * 8]) = st[slot][i];
     };
 
-    // This wavefront's share of U, then the first two blocks of V.
+    // The first two blocks of V, then this wavefront's share of U in the order the
+    // multiplication uses it.  (Completion is counted in issue order: the LDS stores below
+    // wait for V only, and each matrix instruction of the first step only for the filter
+    // fragments up to its own, so the first step starts while most of U is still arriving:
+    // -0.5 us per launch at 64 boards against U first.)
+    gload(0, 0);
+    if (NBLK > 1) gload(1, 1);
     int4v u[NKC];
     {
         const half_t* Up =
@@ -1503,8 +1509,6 @@ __global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restri
         for (int kc = 0; kc < NKC; kc++)
             u[kc] = *reinterpret_cast<const int4v*>(Up + (size_t)kc * 64 * 8);
     }
-    gload(0, 0);
-    if (NBLK > 1) gload(1, 1);
     lstore(0, 0);
     if (NBLK > 1) lstore(1, 1);
     __syncthreads();
@@ -1796,141 +1800,182 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// kHeadPB positions per workgroup share every weight they read.  Thread o owns
-// output o of a fully connected layer and walks the inputs in order, reading
-// the input-major copy of the weights (consecutive threads, consecutive
-// addresses) and the activations as LDS broadcasts; the input range is cut in
-// kHeadSplit pieces taken by separate thread groups, whose partial sums meet in
-// LDS, to shorten the chain of dependent multiply-adds.
-constexpr int kHeadPB = 4;
-constexpr int kHeadGroup = 384;     // >= 362 policy outputs, >= 256 hidden units
-constexpr int kHeadSplit = 2;       // thread groups that share an output's input range
-constexpr int kHeadThreads = kHeadGroup * kHeadSplit;
+// The two large fully connected layers -- policy 722 -> 362 and value 361 -> 256 -- are
+// matrix products over the batch, [n x K] . [K x N], and run on the matrix cores in fp32
+// (v_mfma_f32_32x32x2_f32: fp32 operands, fp32 accumulate).  One work-group computes a
+// 32-position x 32-output tile: the 32 input rows (batch norm and ReLU applied on the way)
+// are staged in LDS once, the four wavefronts split the contraction index four ways, and
+// their partial tiles meet in LDS.  The weights are held in the operand order of the
+// instruction (head_fc_fragments): lane l of k-step s supplies W^T[2s + l/32][32 cb + l%32],
+// four consecutive steps per 16-byte load, so a wavefront's load is one contiguous KiB.
+// A second, small kernel finishes: softmax over the 362 logits, and FC 256 -> 1 + tanh.
+constexpr int kHeadStepsPol = 92;   // k-steps (of 2) per wavefront: 4 * 92 * 2 = 736 >= 722
+constexpr int kHeadStepsVal = 48;   // 4 * 48 * 2 = 384 >= 361
+constexpr int kHeadColsPol = 12;    // 32-wide output blocks: 384 >= 362
+constexpr int kHeadColsVal = 8;     // 256
+constexpr int kHeadKPad = 4 * kHeadStepsPol * 2;   // staged row length of the wider layer
 
-__global__ __launch_bounds__(kHeadThreads) void heads_k(const float* __restrict__ pol,
-                                                        const float* __restrict__ val,
-                                                        HeadParams hp, float temperature,
-                                                        float* __restrict__ policy,
-                                                        float* __restrict__ logits,
-                                                        float* __restrict__ value, int n) {
-    __shared__ float xin[kHeadPB][2 * kPts];
-    __shared__ float part[kHeadSplit][kHeadPB][364];
-    __shared__ float hv[kHeadPB][256];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int grp = tid / kHeadGroup, o = tid - grp * kHeadGroup;   // input range, output
-    const int b0 = blockIdx.x * kHeadPB;
-    const int nb = min(kHeadPB, n - b0);
+size_t head_fc_fragment_count(bool policy) {
+    return (size_t)(policy ? kHeadColsPol * kHeadStepsPol : kHeadColsVal * kHeadStepsVal) * 4 *
+           64;
+}
 
-    // ---- policy: BN + ReLU, FC 722 -> 362, softmax
-    for (int i = tid; i < kHeadPB * 2 * kPts; i += kHeadThreads) {
-        const int pb = i / (2 * kPts), k = i - pb * (2 * kPts), pl = k / kPts;
-        xin[pb][k] = pb < nb ? fmaxf(0.0f, hp.bn_pol_scale[pl] *
-                                               (pol[(size_t)(b0 + pb) * 2 * kPts + k] -
-                                                hp.bn_pol_mean[pl]))
-                             : 0.0f;
-    }
-    __syncthreads();
-    if (o < 362) {
-        float acc[kHeadPB];
+// W [N][K] row-major (as the network facade holds it) -> fragment order
+// [col block][wavefront 4][steps/4][lane 64][4 consecutive steps], zero padded.
+void head_fc_fragments(const float* W, bool policy, float* dst) {
+    const int K = policy ? 2 * kPts : kPts, N = policy ? 362 : 256;
+    const int steps = policy ? kHeadStepsPol : kHeadStepsVal;
+    const int cols = policy ? kHeadColsPol : kHeadColsVal;
+    for (int cb = 0; cb < cols; cb++)
+        for (int q = 0; q < 4; q++)
+            for (int g = 0; g < steps / 4; g++)
+                for (int l = 0; l < 64; l++)
+                    for (int e = 0; e < 4; e++) {
+                        const int step = q * steps + g * 4 + e;
+                        const int k = 2 * step + (l >> 5), j = cb * 32 + (l & 31);
+                        const float v = (k < K && j < N) ? W[(size_t)j * K + k] : 0.0f;
+                        dst[((((size_t)cb * 4 + q) * (steps / 4) + g) * 64 + l) * 4 + e] = v;
+                    }
+}
+
+__global__ __launch_bounds__(256) void heads_fc_k(const float* __restrict__ pol,
+                                                  const float* __restrict__ val, HeadParams hp,
+                                                  float* __restrict__ logits,
+                                                  float* __restrict__ hidden, int n) {
+    constexpr int ROW = kHeadKPad + 1;   // odd row length: conflict-free column reads
+    __shared__ float xs[32 * ROW];
+    const int tasks = kHeadColsPol + kHeadColsVal;
+    const int rb = blockIdx.x / tasks, task = blockIdx.x - rb * tasks;
+    const bool policy = task < kHeadColsPol;
+    const int cb = policy ? task : task - kHeadColsPol;
+    const int K = policy ? 2 * kPts : kPts;
+    const int steps = policy ? kHeadStepsPol : kHeadStepsVal;
+    const int kpad = 4 * steps * 2;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int q = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r0 = rb * 32;
+
+    // the first weight fragments go out before the rows are staged
+    const float4v* wf = reinterpret_cast<const float4v*>(policy ? hp.ip_pol_wf : hp.ip1_val_wf) +
+                        (((size_t)cb * 4 + q) * (steps / 4)) * 64 + lane;
+    constexpr int AHEAD = 6;
+    float4v w[AHEAD];
 #pragma unroll
-        for (int pb = 0; pb < kHeadPB; pb++) acc[pb] = grp == 0 ? hp.ip_pol_b[o] : 0.0f;
-        constexpr int span = 2 * kPts / kHeadSplit;
-        const float* w = hp.ip_pol_wt + (size_t)grp * span * 362 + o;
-#pragma unroll 8
-        for (int k = 0; k < span; k++) {
-            const float wk = w[(size_t)k * 362];
-#pragma unroll
-            for (int pb = 0; pb < kHeadPB; pb++) acc[pb] += wk * xin[pb][grp * span + k];
-        }
-#pragma unroll
-        for (int pb = 0; pb < kHeadPB; pb++) part[grp][pb][o] = acc[pb];
-    }
-    __syncthreads();
-    if (wave < nb) {   // one wavefront per position
-        const int pb = wave;
-        float l[6], m = -INFINITY;
-#pragma unroll
-        for (int q = 0; q < 6; q++) {
-            const int i = lane + 64 * q;
-            l[q] = -INFINITY;
-            if (i < 362) {
-                l[q] = part[0][pb][i];
-#pragma unroll
-                for (int g = 1; g < kHeadSplit; g++) l[q] += part[g][pb][i];
-            }
-            m = fmaxf(m, l[q]);
-        }
-        m = wave_max(m);
-        float e[6];
-        float s = 0.0f;
-#pragma unroll
-        for (int q = 0; q < 6; q++) {
-            e[q] = lane + 64 * q < 362 ? expf((l[q] - m) / temperature) : 0.0f;
-            s += e[q];
-        }
-        s = wave_sum(s);
-#pragma unroll
-        for (int q = 0; q < 6; q++) {
-            const int i = lane + 64 * q;
-            if (i < 362) {
-                policy[(size_t)(b0 + pb) * 362 + i] = e[q] / s;
-                if (logits != nullptr) logits[(size_t)(b0 + pb) * 362 + i] = l[q];
+    for (int g = 0; g < AHEAD; g++) w[g] = wf[(size_t)g * 64];
+
+    // 32 rows of the layer's input: batch norm + ReLU of the raw head planes, zero padded
+    for (int i = tid; i < 32 * kpad; i += 256) {
+        const int r = i / kpad, k = i - r * kpad;
+        float x = 0.0f;
+        if (r0 + r < n && k < K) {
+            if (policy) {
+                const int pl = k >= kPts ? 1 : 0;
+                x = fmaxf(0.0f, hp.bn_pol_scale[pl] *
+                                    (pol[(size_t)(r0 + r) * 2 * kPts + k] - hp.bn_pol_mean[pl]));
+            } else {
+                x = fmaxf(0.0f, hp.bn_val_scale[0] *
+                                    (val[(size_t)(r0 + r) * kPts + k] - hp.bn_val_mean[0]));
             }
         }
+        xs[r * ROW + k] = x;
     }
     __syncthreads();
 
-    // ---- value: BN + ReLU, FC 361 -> 256 + ReLU, FC 256 -> 1, tanh
-    for (int i = tid; i < kHeadPB * kPts; i += kHeadThreads) {
-        const int pb = i / kPts, k = i - pb * kPts;
-        xin[pb][k] = pb < nb ? fmaxf(0.0f, hp.bn_val_scale[0] *
-                                               (val[(size_t)(b0 + pb) * kPts + k] -
-                                                hp.bn_val_mean[0]))
-                             : 0.0f;
-    }
-    __syncthreads();
-    if (o < 256) {
-        float acc[kHeadPB];
+    float16v acc;
 #pragma unroll
-        for (int pb = 0; pb < kHeadPB; pb++) acc[pb] = grp == 0 ? hp.ip1_val_b[o] : 0.0f;
-        // 361 inputs: the first group takes 181, the second 180
-        constexpr int span0 = (kPts + kHeadSplit - 1) / kHeadSplit;
-        const int k0 = grp * span0, k1 = min(kPts, k0 + span0);
-        const float* w = hp.ip1_val_wt + o;
-#pragma unroll 8
-        for (int k = k0; k < k1; k++) {
-            const float wk = w[(size_t)k * 256];
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    const float* xa = xs + (lane & 31) * ROW + q * steps * 2 + (lane >> 5);
+    const int groups = steps / 4;
+    for (int g0 = 0; g0 < groups; g0 += AHEAD) {
 #pragma unroll
-            for (int pb = 0; pb < kHeadPB; pb++) acc[pb] += wk * xin[pb][k];
-        }
-#pragma unroll
-        for (int pb = 0; pb < kHeadPB; pb++) part[grp][pb][o] = acc[pb];
-    }
-    __syncthreads();
-    if (tid < 256) {
-        const float w2 = hp.ip2_val_w[tid];
-#pragma unroll
-        for (int pb = 0; pb < kHeadPB; pb++) {
-            float h = part[0][pb][tid];
-#pragma unroll
-            for (int g = 1; g < kHeadSplit; g++) h += part[g][pb][tid];
-            hv[pb][tid] = fmaxf(0.0f, h) * w2;
+        for (int u = 0; u < AHEAD; u++) {
+            const int g = g0 + u;
+            if (g < groups) {     // uniform
+                const float4v b = w[u];
+                if (g + AHEAD < groups) w[u] = wf[(size_t)(g + AHEAD) * 64];
+                const float* x = xa + g * 8;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[0], b.x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[2], b.y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[4], b.z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[6], b.w, acc, 0, 0, 0);
+            }
         }
     }
+    __syncthreads();   // everyone is done with the staged rows: reuse them for the partial tiles
+
+    // register r of lane l holds row 8(r/4) + 4(l/32) + r%4, column l%32
+    float* red = xs + q * (32 * 33);
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+        red[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 33 + (lane & 31)] = acc[r];
     __syncthreads();
-    if (wave < nb) {
-        const int pb = wave;
-        float acc = 0.0f;
-        for (int i = lane; i < 256; i += 64) acc += hv[pb][i];
-        acc = wave_sum(acc);
-        if (lane == 0) value[b0 + pb] = tanhf(hp.ip2_val_b[0] + acc);
+    const int N = policy ? 362 : 256;
+    for (int i = tid; i < 32 * 32; i += 256) {
+        const int r = i >> 5, j = i & 31;
+        const int col = cb * 32 + j;
+        if (r0 + r < n && col < N) {
+            float v = xs[r * 33 + j] + xs[32 * 33 + r * 33 + j] + xs[2 * 32 * 33 + r * 33 + j] +
+                      xs[3 * 32 * 33 + r * 33 + j];
+            if (policy) {
+                logits[(size_t)(r0 + r) * 362 + col] = v + hp.ip_pol_b[col];
+            } else {
+                hidden[(size_t)(r0 + r) * 256 + col] = fmaxf(0.0f, v + hp.ip1_val_b[col]);
+            }
+        }
     }
 }
 
+// One wavefront per position: softmax over the logits at `temperature`, and the value
+// head's second layer + tanh (reference src/Network.cpp:693-712, :846-851).
+__global__ __launch_bounds__(256) void heads_finish_k(const float* __restrict__ logits_in,
+                                                      const float* __restrict__ hidden,
+                                                      HeadParams hp, float temperature,
+                                                      float* __restrict__ policy,
+                                                      float* __restrict__ logits_out,
+                                                      float* __restrict__ value, int n) {
+    const int pos = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (pos >= n) return;
+    float l[6], m = -INFINITY;
+#pragma unroll
+    for (int qq = 0; qq < 6; qq++) {
+        const int i = lane + 64 * qq;
+        l[qq] = i < 362 ? logits_in[(size_t)pos * 362 + i] : -INFINITY;
+        m = fmaxf(m, l[qq]);
+    }
+    m = wave_max(m);
+    float e[6], s = 0.0f;
+#pragma unroll
+    for (int qq = 0; qq < 6; qq++) {
+        e[qq] = lane + 64 * qq < 362 ? expf((l[qq] - m) / temperature) : 0.0f;
+        s += e[qq];
+    }
+    s = wave_sum(s);
+#pragma unroll
+    for (int qq = 0; qq < 6; qq++) {
+        const int i = lane + 64 * qq;
+        if (i < 362) {
+            policy[(size_t)pos * 362 + i] = e[qq] / s;
+            if (logits_out != nullptr) logits_out[(size_t)pos * 362 + i] = l[qq];
+        }
+    }
+    float acc = 0.0f;
+    for (int i = lane; i < 256; i += 64) acc += hidden[(size_t)pos * 256 + i] * hp.ip2_val_w[i];
+    acc = wave_sum(acc);
+    if (lane == 0) value[pos] = tanhf(hp.ip2_val_b[0] + acc);
+}
+
 void launch_heads(const float* pol, const float* val, HeadParams hp, float temperature,
-                  float* policy, float* logits, float* value, int n, hipStream_t s) {
-    hipLaunchKernelGGL(heads_k, dim3((n + kHeadPB - 1) / kHeadPB), dim3(kHeadThreads), 0, s, pol,
-                       val, hp, temperature, policy, logits, value, n);
+                  float* policy, float* logits, float* value, float* work, int n,
+                  hipStream_t s) {
+    // work: [n][362] logits followed by [n][256] hidden units
+    float* wl = work;
+    float* wh = work + (size_t)n * 362;
+    const int rbs = (n + 31) / 32;
+    hipLaunchKernelGGL(heads_fc_k, dim3(rbs * (kHeadColsPol + kHeadColsVal)), dim3(256), 0, s, pol,
+                       val, hp, wl, wh, n);
+    hipLaunchKernelGGL(heads_finish_k, dim3((n + 3) / 4), dim3(256), 0, s, wl, wh, hp, temperature,
+                       policy, logits, value, n);
 }
 
 // ---------------------------------------------------------------------------
