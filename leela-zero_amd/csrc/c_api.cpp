@@ -86,9 +86,16 @@ int lzhip_create_from_file(const char* path, int precision, int max_batch, int d
     const WeightsFile wf = load_weights_file(path);   // before any device is touched
     if (filters) *filters = wf.filters;
     if (blocks) *blocks = wf.blocks;
-    lzhip_handle* h = nullptr;
-    int rc = lzhip_create(wf.filters, precision, max_batch, device, &h);
+    lzhip_handle* raw = nullptr;
+    int rc = lzhip_create(wf.filters, precision, max_batch, device, &raw);
     if (rc != LZHIP_OK) return rc;
+    // owned until everything has succeeded: an exception below (e.g. bad_alloc in the
+    // pointer tables) must not leave the handle behind
+    struct Destroy {
+        void operator()(lzhip_handle* p) const { delete p; }
+    };
+    std::unique_ptr<lzhip_handle, Destroy> owner(raw);
+    lzhip_handle* h = raw;
     const size_t nl = wf.U.size();
     std::vector<const float*> U(nl), mean(nl), scale(nl);
     for (size_t l = 0; l < nl; l++) {
@@ -105,10 +112,11 @@ int lzhip_create_from_file(const char* path, int precision, int max_batch, int d
                               wf.ip2_val_b.data());
     if (rc != LZHIP_OK) {
         const std::string keep = g_err;
-        lzhip_destroy(h);
+        owner.reset();
         g_err = keep;
         return rc;
     }
+    owner.release();
     h->value_not_stm.store(wf.value_head_not_stm);
     *out = h;
     return LZHIP_OK;

@@ -1416,7 +1416,7 @@ __global__ __launch_bounds__(512) void wino_gemm_split_k(const P* __restrict__ V
 // Uf layout ("fragment order"): [36][Kp/32][Cp/16][64 lanes][8 halves]; lane l of
 // fragment (p, wb, kc) holds U_p[32 wb + gemm_stream_channel(l % 32)][16 kc + 8 (l / 32) + 0..7],
 // so every operand load of a wavefront is one contiguous KiB.
-constexpr int kStreamBlocks = 8;   // most 32-row blocks per work-group (steps of the pipeline)
+constexpr int kStreamBlocks = 16;  // most 32-row blocks per work-group (steps of the pipeline)
 constexpr int kStreamAhead = 2;    // blocks requested ahead of the one being multiplied
 
 __host__ __device__ constexpr int gemm_stream_channel(int i) {
@@ -1606,7 +1606,7 @@ void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, half_t
 
 // Blocks per work-group for T tile rows: the fewest (a power of two up to kStreamBlocks)
 // with which one round of work-groups covers the 256 compute units, so that a batch of 8
-// boards runs one block per work-group and 64 boards eight.
+// boards runs one block per work-group, 64 boards eight and 128 boards sixteen.
 static int gemm_stream_blocks(int T, int Kp) {
     const int nblk = (T + 31) / 32;
     const int per_pos = 256 / (kPos * (Kp / 256));           // work-groups per position in one round
@@ -1636,7 +1636,8 @@ static void launch_gemm_stream_nkc(const half_t* V, const half_t* Uf, half_t* M,
         case 1: launch(wino_gemm_stream_k<NKC, 1>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
         case 2: launch(wino_gemm_stream_k<NKC, 2>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
         case 4: launch(wino_gemm_stream_k<NKC, 4>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        default: launch(wino_gemm_stream_k<NKC, 8>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        case 8: launch(wino_gemm_stream_k<NKC, 8>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        default: launch(wino_gemm_stream_k<NKC, 16>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
     }
 }
 

@@ -149,8 +149,8 @@ def test_forward_parity(pkg, netgen, orc, blocks, filters, batch, precision):
 @pytest.mark.parametrize("batch", [72, 64, 52, 41, 36, 35, 33, 24, 21, 18, 17, 10, 9, 8, 2])
 def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
     """256 filters at batch sizes on both sides of every change of kernel shape (GEMM, fp16:
-    the streaming kernel with 1, 2, 4 and 8 blocks of 32 tile rows per work-group, which
-    change at 9, 18 and 36 boards, and more than one round of work-groups at 72; fp32:
+    the streaming kernel with 1, 2, 4, 8 and 16 blocks of 32 tile rows per work-group, which
+    change at 9, 18, 36 and 72 boards; fp32:
     256x256 tiles from 41 boards, 128x128 from 21, 128x64 with padded rows below; fused
     transform: 64 channels per work-group from 33 boards, 32 from 6, 16 below), in both
     precisions, including batches whose tile count is not a multiple of any tile height."""
