@@ -418,6 +418,49 @@ def side_config(pkg, netgen, torch, blocks, F, precision, B, args, cpu=False):
     return out
 
 
+def latency_by_batch(pkg, netgen, torch, blocks, F, precision, args):
+    """Forward latency of the headline network at small batches (one lane, device-resident
+    inputs, median of three runs of 60 forwards), and at batch 16 -- the batch a search with
+    16 threads forms -- also with the forward's launches replayed from a HIP graph."""
+    prec = pkg.FP16 if precision == "fp16" else pkg.FP32
+    net = netgen.make_network(blocks, F, seed=2025)
+    w, _ = netgen.prepare(net)
+    out = {}
+
+    def run(B, graph):
+        if graph:
+            os.environ["LZHIP_GRAPH"] = "1"
+        try:
+            pipe = pkg.HIPScheduler(prec, B, device=0)
+            pipe.initialize(F)
+            pipe.push_weights(6, 18, F, w)
+        finally:
+            os.environ.pop("LZHIP_GRAPH", None)
+        d_in = torch.from_numpy(netgen.synthetic_inputs(B, seed=2026)).cuda()
+        d_pol = torch.zeros(B, 722, device="cuda")
+        d_val = torch.zeros(B, 361, device="cuda")
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(3):
+            for _ in range(10):
+                pipe.forward_batch_device(B, d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
+            pipe.sync()
+            t0 = time.perf_counter()
+            for _ in range(60):
+                pipe.forward_batch_device(B, d_in.data_ptr(), d_pol.data_ptr(), d_val.data_ptr())
+            pipe.sync()
+            ts.append((time.perf_counter() - t0) / 60 * 1e3)
+        pipe.close()
+        return sorted(ts)[1]
+
+    for B in (1, 4, 8, 16, 32):
+        out["b%d_ms" % B] = run(B, False)
+    out["b16_graph_replay_ms"] = run(16, True)
+    out["note"] = ("one lane, ms per forward of the whole batch; graph replay = the same launches "
+                   "captured once and replayed (LZHIP_GRAPH=1)")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -523,6 +566,8 @@ def main():
         # the same network in fp32, and the three smaller configurations, one line each
         if args.precision == "fp16":
             out["fp32"] = side_config(pkg, netgen, torch, blocks, F, "fp32", B, args)
+        out["latency_by_batch"] = latency_by_batch(pkg, netgen, torch, blocks, F, args.precision,
+                                                   args)
         out["configs"] = {
             "6x128 fp32 b1": side_config(pkg, netgen, torch, 6, 128, "fp32", 1, args, cpu=True),
             "15x192 fp32 b8": side_config(pkg, netgen, torch, 15, 192, "fp32", 8, args),

@@ -59,6 +59,8 @@ def test_forward_line():
     for c in d["configs"].values():
         assert c["value"] > 0 and c["one_lane"] > 0
     assert d["configs"]["6x128 fp32 b1"]["cpu_oracle"]["value"] > 0
+    lb = d["latency_by_batch"]
+    assert 0 < lb["b1_ms"] <= lb["b32_ms"] and lb["b16_graph_replay_ms"] > 0
 
 
 def test_more_than_one_gpu_is_refused():
