@@ -465,9 +465,17 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     constexpr int TPW = 64 / CP;      // tiles per wavefront
     constexpr int WAVES = fuse_waves(CG);
     __shared__ pair_t ybuf[kPlane * kPlane * CP];
+    // Work-group w runs on die w % 8, each die with its own L2.  The narrow shapes share
+    // 128-byte lines between the work-groups of neighbouring channel groups, so the items
+    // (board, channel group) are cut into 8 contiguous segments and work-group w takes item
+    // w / 8 of segment w % 8: the sharers then sit on one die and a line comes from memory
+    // once, instead of once for each die that holds a piece of it.
     const int ncg = Kp / CG;
-    const int b = blockIdx.x / ncg;
-    const int cg = blockIdx.x - b * ncg;
+    const int per_die = (n * ncg + 7) >> 3;
+    const int item = (int)(blockIdx.x & 7) * per_die + (int)(blockIdx.x >> 3);
+    if (item >= n * ncg) return;
+    const int b = item / ncg;
+    const int cg = item - b * ncg;
 
     const unsigned lane = threadIdx.x & 63;
     const unsigned cl = lane % CP, sub = lane / CP;    // channel pair, tile within the wavefront
@@ -655,19 +663,23 @@ template <typename P>
 void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
                              const float* bn_mean, float rfac, int n, int Kp, int Tp,
                              hipStream_t s, LaunchTimer* t) {
-    // 32 channels per work-group for as long as those work-groups fit the 256 compute units
-    // in one go (a board's arithmetic then spreads over twice as many units), 64 beyond
-    // that (measured at 256 filters: 32 wins up to batch 32, 64 from batch 33, by 6 %); 16 only
-    // for the smallest batches (a wash between batch 6 and 12, a loss at 8 and 16).
+    // The narrowest shape whose work-groups fit the 256 compute units in one go: a board's
+    // arithmetic then spreads over the most units (measured at 256 filters, per launch:
+    // 16 channels 7.7 us against 8.4 with 32 and 9.7 with 64 at batch 16; 32 channels 10.1
+    // against 10.4 with 64 and 11.0 with 16 at batch 32; 64 channels from batch 33: 10.5
+    // against 13.0 at 36).  The narrow shapes only pay with the die-aware item order of the
+    // kernel: dealt round-robin over the dies, their work-groups fetch every line of M once
+    // per die that holds a piece of it (16 channels at batch 16: 11.2 us).
     const int items64 = n * (Kp / 64);
+    auto grid = [](int items) { return dim3((unsigned)(8 * ((items + 7) / 8))); };
     if (items64 > 128)
-        launch(out_in_transform_k<P, 64>, dim3(items64), dim3(fuse_waves(64) * 64), s, t, M, res,
+        launch(out_in_transform_k<P, 64>, grid(items64), dim3(fuse_waves(64) * 64), s, t, M, res,
                act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
-    else if (items64 >= 24)
-        launch(out_in_transform_k<P, 32>, dim3(items64 * 2), dim3(fuse_waves(32) * 64), s, t, M,
+    else if (items64 > 64)
+        launch(out_in_transform_k<P, 32>, grid(items64 * 2), dim3(fuse_waves(32) * 64), s, t, M,
                res, act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
     else
-        launch(out_in_transform_k<P, 16>, dim3(items64 * 4), dim3(fuse_waves(16) * 64), s, t, M,
+        launch(out_in_transform_k<P, 16>, grid(items64 * 4), dim3(fuse_waves(16) * 64), s, t, M,
                res, act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
 }
 
