@@ -79,11 +79,15 @@ def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None, all_raw=Fa
     most one position of a case may take that route.  Raw planes and logits are always
     compared at the strict relative tolerance, for every position checked; with all_raw
     the raw planes of every position of the batch are (the oracle runs them on all host
-    threads), whatever idx selects for the head outputs."""
+    threads), whatever idx selects for the head outputs.  Every position checked must also
+    pass the engine's own run-time self-check (Network::compare_net_outputs, reference
+    src/Network.cpp:666-691): the L2 norm over the 362 policy entries and the winrate
+    (1 + value) / 2 at most 0.2, with no relaxation for ill-conditioned positions."""
     raw_tol = 1e-5 if precision == 0 else 2e-2
     p_tol = 1e-4 if precision == 0 else 2e-2
     policy, value, logits, pol, val = pipe.evaluate_batch(x, want_raw=True)
-    worst = dict(pol=0.0, val=0.0, logits=0.0, policy=0.0, value=0.0, ill_conditioned=0)
+    worst = dict(pol=0.0, val=0.0, logits=0.0, policy=0.0, value=0.0, ill_conditioned=0,
+                 engine_selfcheck=0.0)
     if all_raw:
         import os
         rp_all, rv_all, _ = ref.forward_many(x, threads=min(16, os.cpu_count() or 1))
@@ -121,6 +125,10 @@ def check_outputs(pkg, orc, pipe, ref, h_ref, x, precision, idx=None, all_raw=Fa
         worst["policy"] = max(worst["policy"], e_p)
         worst["value"] = max(worst["value"], e_v)
         assert e_p <= tol_i and e_v <= tol_i, (i, e_p, e_v, tol_i)
+        d = np.asarray(policy[i], np.float64) - np.asarray(hd["policy"], np.float64)
+        e_engine = float(np.sqrt(np.sum(d * d) + (0.5 * (float(value[i]) - hd["value"])) ** 2))
+        worst["engine_selfcheck"] = max(worst["engine_selfcheck"], e_engine)
+        assert e_engine <= 0.2, ("engine self-check bar", i, e_engine)
         assert abs(float(policy[i].sum()) - 1.0) < 1e-4
     print("parity", worst, flush=True)
     assert worst["pol"] <= raw_tol and worst["val"] <= raw_tol, worst
