@@ -1399,14 +1399,15 @@ __global__ __launch_bounds__(512) void wino_gemm_split_k(const P* __restrict__ V
 }
 
 // ---------------------------------------------------------------------------
-// Filter-stationary streaming GEMM (fp16 storage).  One work-group of 8 wavefronts
-// owns one Winograd position and a run of consecutive 32-row blocks of V; wavefront
-// w owns output channels 32w..32w+31 of a 256-channel column tile and keeps its
+// Filter-stationary streaming GEMM (fp16 storage).  One work-group of NW wavefronts
+// (8 at 256 filters, 6 / 4 / 2 at 192 / 128 / 64) owns one Winograd position and a run of
+// consecutive 32-row blocks of V; wavefront w owns output channels 32w..32w+31 of a
+// column tile of 32 NW channels and keeps its
 // share of U_p -- 32 channels x Cp input channels -- in registers for the whole
 // kernel (Cp/4 registers per lane), already in the order the matrix instruction
 // wants it.  V streams through: a 32-row block (all Cp input channels, so the
 // contraction of those rows completes in one step) is requested kStreamAhead steps
-// ahead into registers and passes through a three-stage LDS ring, where all eight
+// ahead into registers and passes through a three-stage LDS ring, where all
 // wavefronts read it as their column operand.  A step multiplies one block; the
 // fragment reads of the block's second half and of the next block's first half are
 // issued ahead of the matrix instructions that hide them, and one barrier ends the
@@ -1417,8 +1418,8 @@ __global__ __launch_bounds__(512) void wino_gemm_split_k(const P* __restrict__ V
 // of the row operand.  The row operand is U, and the host stores U's channels permuted
 // (gemm_stream_channel) so that this lane's sixteen registers are the channels
 // 16(r/8) + 8(l/32) + r%8 of the wavefront's 32, i.e. two 16-byte runs.  Those go into
-// an LDS copy of the block's 32 x 256 result, and one step later (behind the barrier
-// that is there anyway) every wavefront sends four whole rows of it, 1 KiB per store
+// an LDS copy of the block's 32 x 32 NW result, and one step later (behind the barrier
+// that is there anyway) every wavefront sends its share of the rows, 1 KiB per store
 // instruction.  The stores are write-through (sc0 sc1): whole lines leave for memory
 // while the kernel runs, instead of collecting as dirty lines in the L2 that the end
 // of the kernel has to flush with nothing else in flight (measured at 64 boards and
@@ -1436,22 +1437,24 @@ __host__ __device__ constexpr int gemm_stream_channel(int i) {
     return 16 * (i >> 4) + 8 * ((i >> 2) & 1) + 4 * ((i >> 3) & 1) + (i & 3);
 }
 
-template <int NKC, int NBLK>
-__global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restrict__ V,
+template <int NKC, int NBLK, int NW>
+__global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __restrict__ V,
                                                           const half_t* __restrict__ Uf,
                                                           half_t* __restrict__ M, int T, int Tp,
                                                           int Kp, int chunks, int nblk_total,
                                                           int tiles_n, int seg) {
     constexpr int D = kStreamAhead;
+    constexpr int NT = 64 * NW;                  // threads: NW wavefronts of 32 output channels
+    constexpr int CW = 32 * NW;                  // width of the column tile
     constexpr int Cp = NKC * 16;
     constexpr int HK = NKC / 2;                  // fragments per half block
     constexpr int CPRW = Cp / 8;                 // 16-byte chunks per row
     constexpr int NCH = 32 * CPRW;               // chunks per block
-    constexpr int CH = (NCH + 511) / 512;        // chunk loads per thread and block
-    constexpr bool FULL = NCH % 512 == 0;        // every thread has all CH chunks
+    constexpr int CH = (NCH + NT - 1) / NT;      // chunk loads per thread and block
+    constexpr bool FULL = NCH % NT == 0;         // every thread has all CH chunks
     constexpr int ROWE = Cp + 8;                 // padded LDS row (halves): conflict-free 16-byte reads
     constexpr int STAGE = 32 * ROWE;
-    constexpr int OROW = 256 + 8;                // row of the output copy (halves)
+    constexpr int OROW = CW + 8;                 // row of the output copy (halves)
     constexpr int OSTAGE = 32 * OROW;
     static_assert(NKC % 2 == 0 && D == 2, "pipeline shape");
 
@@ -1480,7 +1483,7 @@ __global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restri
     bool lval[CH];
 #pragma unroll
     for (int i = 0; i < CH; i++) {
-        const int idx = tid + i * 512;
+        const int idx = tid + i * NT;
         lval[i] = FULL || idx < NCH;
         lrow[i] = (idx / CPRW) & 31;
         lcc[i] = idx % CPRW;
@@ -1516,7 +1519,7 @@ __global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restri
     int4v u[NKC];
     {
         const half_t* Up =
-            Uf + ((((size_t)p * (Kp / 32) + (size_t)tn * 8 + wave) * NKC) * 64 + lane) * 8;
+            Uf + ((((size_t)p * (Kp / 32) + (size_t)tn * NW + wave) * NKC) * 64 + lane) * 8;
 #pragma unroll
         for (int kc = 0; kc < NKC; kc++)
             u[kc] = *reinterpret_cast<const int4v*>(Up + (size_t)kc * 64 * 8);
@@ -1533,16 +1536,28 @@ __global__ __launch_bounds__(512) void wino_gemm_stream_k(const half_t* __restri
     const size_t m_bytes = (size_t)T * Kp * sizeof(half_t);
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(M + (size_t)p * Tp * Kp, m_bytes);
     const unsigned m_rowb = (unsigned)Kp * 2u;
-    const unsigned m_col = (unsigned)(tn * 256 + jrow * 8) * 2u;
-    // wavefront w sends rows 4w..4w+3 of a block: two whole rows per store instruction
+    // The 32 x CW result leaves in 16-byte pieces, two per thread.  Eight wavefronts:
+    // wavefront w sends rows 4w..4w+3, two whole 512-byte rows per store instruction.  Fewer:
+    // the pieces are dealt to the threads in memory order (a row holds CW / 8 of them), so
+    // that a store instruction still writes one contiguous KiB when the tile is the whole row.
+    constexpr int PPR = CW / 8;
     auto send_rows = [&](int s) {
         const half_t* O = obuf + (s & 1) * OSTAGE;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const int r = wave * 4 + hh + 2 * i;
-            const int4v v = *reinterpret_cast<const int4v*>(O + r * OROW + jrow * 8);
+            int r, cc;
+            if constexpr (NW == 8) {
+                r = wave * 4 + hh + 2 * i;
+                cc = jrow;
+            } else {
+                const int piece = tid + i * NT;
+                r = piece / PPR;
+                cc = piece - r * PPR;
+            }
+            const int4v v = *reinterpret_cast<const int4v*>(O + r * OROW + cc * 8);
             const unsigned row = (unsigned)((blk0 + s) * 32 + r);
-            const unsigned vo = s < nreal ? row * m_rowb + m_col : 0x7ffffff0u;
+            const unsigned vo =
+                s < nreal ? row * m_rowb + (unsigned)(tn * CW + cc * 8) * 2u : 0x7ffffff0u;
             __builtin_amdgcn_raw_buffer_store_b128(v, rM, vo, 0, kStoreThrough);
         }
     };
@@ -1621,44 +1636,58 @@ void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, half_t
 // boards runs one block per work-group, 64 boards eight and 128 boards sixteen.
 static int gemm_stream_blocks(int T, int Kp) {
     const int nblk = (T + 31) / 32;
-    const int per_pos = 256 / (kPos * (Kp / 256));           // work-groups per position in one round
+    const int per_pos = 256 / (kPos * ((Kp + 255) / 256));   // work-groups per position in one round
     int nb = 1;
     while (nb < kStreamBlocks && (nblk + nb - 1) / nb > per_pos) nb *= 2;
     return nb;
 }
 
 // Whether launch_gemm takes the streaming kernel for this shape (the caller then has to
-// hold the fragment-order filters): fp16 nets of 256 filters, any batch.
+// hold the fragment-order filters): fp16 nets of 128, 192 and 256 filters (one column tile
+// of Kp / 32 wavefronts), input layer (64 padded planes) and tower layers, any batch.
+// (At 64 filters the tiled kernel is as fast: measured 3.0 against 3.5 us at 4 boards, 3.5
+// against 3.5 at 33.)
 bool gemm_stream_shape(int T, int Cp, int Kp) {
-    return T >= 1 && Kp == 256 && (Cp == 64 || Cp == 256);
+    return T >= 1 && (Kp == 128 || Kp == 192 || Kp == 256) && (Cp == 64 || Cp == Kp);
 }
 
-template <int NKC>
+template <int NKC, int NW>
 static void launch_gemm_stream_nkc(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
                                    int Kp, hipStream_t s, LaunchTimer* t) {
     const int nblk = (T + 31) / 32;
     const int nb = gemm_stream_blocks(T, Kp);
     const int chunks = (nblk + nb - 1) / nb;
-    const int tiles_n = Kp / 256;
+    const int tiles_n = Kp / (32 * NW);
     const int n_items = kPos * chunks * tiles_n;
     int seg = (n_items + 7) / 8;
     seg = (seg + tiles_n - 1) / tiles_n * tiles_n;
-    const dim3 grid(8 * seg), block(512);
+    const dim3 grid(8 * seg), block(64 * NW);
     switch (nb) {
-        case 1: launch(wino_gemm_stream_k<NKC, 1>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        case 2: launch(wino_gemm_stream_k<NKC, 2>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        case 4: launch(wino_gemm_stream_k<NKC, 4>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        case 8: launch(wino_gemm_stream_k<NKC, 8>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        default: launch(wino_gemm_stream_k<NKC, 16>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        case 1: launch(wino_gemm_stream_k<NKC, 1, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        case 2: launch(wino_gemm_stream_k<NKC, 2, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        case 4: launch(wino_gemm_stream_k<NKC, 4, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        case 8: launch(wino_gemm_stream_k<NKC, 8, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+        default: launch(wino_gemm_stream_k<NKC, 16, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
     }
+}
+
+// NW = Kp / 32 wavefronts per work-group; the first layer reads the 64 padded input planes.
+template <int NW>
+static void launch_gemm_stream_nw(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
+                                  int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
+    if (Cp == 64)
+        launch_gemm_stream_nkc<4, NW>(V, Uf, M, T, Tp, Kp, s, t);
+    else
+        launch_gemm_stream_nkc<2 * NW, NW>(V, Uf, M, T, Tp, Kp, s, t);
 }
 
 static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
                                int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
-    if (Cp == 256)
-        launch_gemm_stream_nkc<16>(V, Uf, M, T, Tp, Kp, s, t);
-    else
-        launch_gemm_stream_nkc<4>(V, Uf, M, T, Tp, Kp, s, t);
+    switch (Kp) {
+        case 256: launch_gemm_stream_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
+        case 192: launch_gemm_stream_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
+        default: launch_gemm_stream_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
+    }
 }
 
 template <typename P, int NK>

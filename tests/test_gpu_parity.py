@@ -507,13 +507,28 @@ def test_error_behaviour_on_device(pkg, netgen):
         p.initialize(64)
 
 
+@pytest.mark.parametrize("filters,batch", [(128, 1), (128, 9), (128, 30), (128, 52), (128, 72),
+                                           (192, 2), (192, 17), (192, 40), (192, 64)])
+def test_fp16_streaming_gemm_at_narrower_widths(pkg, netgen, orc, filters, batch):
+    """fp16 nets of 128 and 192 filters run the streaming GEMM with 4 and 6 wavefronts per
+    work-group (256 filters: 8); the batches take every number of blocks per work-group
+    (1, 2, 4, 8, 16), with tile counts that are not multiples of the 32-row block."""
+    print("case: fp16 streaming width %d b%d" % (filters, batch), flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, filters, 5100 + filters, pkg.FP16,
+                                       batch)
+    x = netgen.synthetic_inputs(batch, seed=filters + batch)
+    check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16,
+                  idx=sorted({0, batch // 2, batch - 1}))
+    pipe.close()
+
+
 @pytest.mark.parametrize("filters,batch", [(640, 4), (768, 3), (896, 2), (1024, 12), (1024, 8),
-                                           (384, 28), (128, 30), (192, 52)])
+                                           (384, 28), (448, 30), (320, 52)])
 def test_fp16_widths_on_the_tiled_gemm(pkg, netgen, orc, filters, batch):
-    """fp16 widths served by the tiled GEMM kernels (every width but 256): the widest ones --
-    10, 12, 14 and 16 k-slices, at 1024 filters the one-pass 256x256 tile (from 11 boards)
-    and the 128x64 tile below it -- and narrow nets at batches that take the 128x128
-    persistent and the 128x64 tiles."""
+    """fp16 widths served by the tiled GEMM kernels (above 256 filters; 64-filter nets are in
+    the small-network cases): the widest ones -- 10, 12, 14 and 16 k-slices, at 1024 filters
+    the one-pass 256x256 tile (from 11 boards) and the 128x64 tile below it -- and widths
+    at batches that take the 128x128 persistent and the 128x64 tiles."""
     print("case: fp16 width %d b%d" % (filters, batch), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, filters, 5000 + filters, pkg.FP16,
                                        batch)
