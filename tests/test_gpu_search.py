@@ -268,7 +268,7 @@ def test_value_head_of_format_2_networks(pkg, netgen, orc, tmp_path):
 
 
 def test_search_configuration_four_at_full_size(pkg, netgen):
-    """BASELINE configs[4] as written: 16 search threads, max batch 32, the 40x256 fp16
+    """The search benchmark configuration at full size: 16 search threads, max batch 32, the 40x256 fp16
     network, 1600 visits per move, 20 moves from the empty board (the call pattern of the
     reference's UCTSearch::think, src/UCTSearch.cpp:757-850, threads/batch defaults
     src/Leela.cpp:64-133).  The fully connected head weights are rescaled as bench.py does
