@@ -340,6 +340,19 @@ def measure_forward(pkg, netgen, torch, blocks, F, precision, B, steps, warmup, 
     }
     roofline["launch_context"] = ("launches that run alone (event-timed forward on one lane, "
                                   "nothing else enqueued)")
+    # The events bracket a launch's own execution; what lies between two launches of a chain
+    # (the hand-over from one kernel to the next) is not in them, and a kernel trace, whose
+    # durations run from one dispatch to the next, reads longer by that much.  The same
+    # forward priced launch to launch: the one-lane wall time shared out over the launches
+    # in proportion to their event durations.
+    wall_ms = res["one_lane"]["ms_per_step"]
+    stretch = wall_ms / float(ms.sum())
+    roofline["launch_to_launch"] = {
+        "avg_launch_us": roofline["avg_launch_us"] * stretch,
+        "frac": roofline["frac"] / stretch,
+        "note": "one-lane forward wall time (%.3f ms) shared out over its %d launches in "
+                "proportion to their event durations: what a kernel trace reads per launch"
+                % (wall_ms, int(cnt.sum()))}
     if ms2 is not None:
         roofline["side_by_side"] = {
             "avg_launch_us": ms2[pkg.K_GEMM] * 1e3 / cnt[pkg.K_GEMM],

@@ -38,6 +38,9 @@ def test_forward_line():
         assert k in rf, k
     assert rf["bound"] == "mfma" and rf["unit"] == "TFLOP/s" and 0 < rf["frac"] < 1
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
+    # the same launch priced launch to launch (what a kernel trace reads) is the longer one
+    l2l = rf["launch_to_launch"]
+    assert l2l["avg_launch_us"] >= rf["avg_launch_us"] and 0 < l2l["frac"] <= rf["frac"]
     cb = d["cpu_baseline"]
     for k in ("value", "unit", "cores", "kind", "sample"):
         assert k in cb, k
