@@ -244,15 +244,13 @@ public:
                 }
             L.U.alloc(tmp.size());
             HIP_CHECK(hipMemcpy(L.U.p, tmp.data(), tmp.size() * sizeof(P), hipMemcpyHostToDevice));
-            // Second copy in the fragment order of the streaming GEMM, where the largest
-            // batch of this handle can take that kernel.
-            if constexpr (sizeof(P) == 2) {
-                if (gemm_stream_shape(m_max_batch * kTilesPerBoard, L.Cp, m_Fp)) {
-                    build_stream_filters(U[l], L.C, F, L.Cp, m_Fp, tmp.data());
-                    L.Uf.alloc(tmp.size());
-                    HIP_CHECK(hipMemcpy(L.Uf.p, tmp.data(), tmp.size() * sizeof(P),
-                                        hipMemcpyHostToDevice));
-                }
+            // Second copy in the fragment order of the streaming GEMM, where some batch of
+            // this handle can take that kernel (the smallest does if any).
+            if (gemm_stream_shape(kTilesPerBoard, L.Cp, m_Fp, (int)sizeof(P))) {
+                build_stream_filters(U[l], L.C, F, L.Cp, m_Fp, tmp.data());
+                L.Uf.alloc(tmp.size());
+                HIP_CHECK(hipMemcpy(L.Uf.p, tmp.data(), tmp.size() * sizeof(P),
+                                    hipMemcpyHostToDevice));
             }
             L.mean.assign(bn_mean[l], bn_mean[l] + F);
             L.scale.assign(bn_scale[l], bn_scale[l] + F);

@@ -53,14 +53,16 @@ template <typename P> bool gemm_supports_channels(int Cp);
 
 // M[p][t][k] = sum_c V[p][t][c] * U[p][k][c]
 // T = real tile rows (25 per board); Tp = allocated rows, a multiple of kTileRowPad.
-// Uf: the same filters in the fragment order of the streaming kernel (fp16 only, see
-// build_stream_filters), or null; taken when gemm_stream_shape(T, Cp, Kp).
+// Uf: the same filters in the fragment order of the streaming kernels (see
+// build_stream_filters), or null; taken when gemm_stream_shape(T, Cp, Kp, sizeof(P)).
 template <typename P>
 void launch_gemm(const P* V, const P* U, const P* Uf, P* M, int T, int Tp, int Cp, int Kp,
                  hipStream_t s, LaunchTimer* t);
-bool gemm_stream_shape(int T, int Cp, int Kp);
+bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes);
 // src [36][C][F] fp32 (F fastest) -> dst [36][Kp/32][Cp/16][64][8] fp16, zero padded.
 void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, _Float16* dst);
+// ... -> dst [36][Kp/32][Cp/8][64][4] fp32 for the fp32 streaming kernel.
+void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, float* dst);
 
 // M [36][Tp][Kp] -> out [n][361][Kp]:  max(0, scale*(A^T m A - mean) + rfac*res)
 template <typename P>

@@ -1567,6 +1567,10 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
 #pragma unroll
     for (int kc = 0; kc < HK; kc++) alo[kc] = *reinterpret_cast<const int4v*>(smem + frag + kc * 16);
 
+    // Every work-group runs all NBLK steps; those past its last block multiply stale data and
+    // store nothing.  (Leaving after nreal steps, with the blocks split evenly over 7
+    // work-groups per position at every batch, was measured and is slower in this kernel,
+    // which the stream bounds: one lane -1 % at 64 boards, -6 % at 96, +5 % at 40.)
 #pragma unroll
     for (int s = 0; s < NBLK; s++) {
         if (s + D < NBLK) gload(s % D, s + D);
@@ -1613,6 +1617,170 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
     send_rows(NBLK - 1);
 }
 
+// ---------------------------------------------------------------------------
+// The same filter-stationary structure in fp32 (v_mfma_f32_32x32x2_f32, a sixteenth of
+// the fp16 matrix rate: this kernel is bound by the matrix pipe, not by the stream).
+// Wavefront w keeps U_p for its 32 output channels in Cp/2 registers per lane; a step
+// multiplies one 32-row block of V, 4 matrix instructions per 16-byte fragment read, so
+// that nothing but the matrix pipe is busy for long.  The contraction index is dealt so
+// that one 16-byte read serves four instructions: in instruction 4j + i, lanes 0..31
+// hold input channel 8j + i and lanes 32..63 channel 8j + 4 + i, of U (rows) and of V
+// (columns) alike.  The block's result goes through a single LDS copy (two barriers per
+// step are little beside 128 matrix instructions) and leaves as whole rows, written
+// through, as in the fp16 kernel.  (Stored straight from the accumulators instead, 64
+// bytes per lane with write-back stores and one barrier per step, the kernel is slower:
+// 87 against 83 us per launch at 64 boards and 256 filters, 28 against 24 at 128 filters.)
+//
+// Uf layout: [36][Kp/32][Cp/8][64 lanes][4 floats]; lane l of fragment (p, wb, j) holds
+// U_p[32 wb + gemm_stream_channel(l % 32)][8 j + 4 (l / 32) + 0..3].
+
+template <int NK8, int NBLK, int NW>
+__global__ __launch_bounds__(64 * NW) void wino_gemm_stream32_k(const float* __restrict__ V,
+                                                                const float* __restrict__ Uf,
+                                                                float* __restrict__ M, int T,
+                                                                int Tp, int Kp, int chunks,
+                                                                int nblk_total, int seg) {
+    constexpr int D = kStreamAhead;
+    constexpr int NT = 64 * NW;
+    constexpr int CW = 32 * NW;
+    constexpr int Cp = NK8 * 8;
+    constexpr int CPRW = Cp / 4;                 // 16-byte chunks per row
+    constexpr int NCH = 32 * CPRW;               // chunks per block
+    constexpr int CH = (NCH + NT - 1) / NT;
+    constexpr bool FULL = NCH % NT == 0;
+    constexpr int ROWE = Cp + 4;                 // padded LDS row (floats)
+    constexpr int STAGE = 32 * ROWE;
+    constexpr int OROW = CW + 4;
+    static_assert(D == 2, "pipeline shape");
+
+    __shared__ __attribute__((aligned(16))) float smem[3 * STAGE + 32 * OROW];
+    float* const obuf = smem + 3 * STAGE;
+
+    const int n_items = kPos * chunks;
+    const int xcd = blockIdx.x & 7;
+    const int item = xcd * seg + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= seg || item >= n_items) return;
+    const int ch = item % chunks;
+    const int p = item / chunks;
+    const int blk0 = (ch * nblk_total) / chunks;
+    const int blk1 = ((ch + 1) * nblk_total) / chunks;
+    const int nreal = blk1 - blk0;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hh = lane >> 5, jrow = lane & 31;
+
+    int lrow[CH], lcc[CH];
+    bool lval[CH];
+#pragma unroll
+    for (int i = 0; i < CH; i++) {
+        const int idx = tid + i * NT;
+        lval[i] = FULL || idx < NCH;
+        lrow[i] = (idx / CPRW) & 31;
+        lcc[i] = idx % CPRW;
+    }
+    const float* Vp = V + (size_t)p * Tp * Cp;
+
+    int4v st[D][CH];
+    auto gload = [&](int slot, int s) {
+        // requests past the last real block re-read that block (cache hits, never used)
+        const int blk = blk0 + (s < nreal ? s : nreal - 1);
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int row = min(blk * 32 + lrow[i], T - 1);
+            if (lval[i])
+                st[slot][i] =
+                    *reinterpret_cast<const int4v*>(Vp + (size_t)row * Cp + lcc[i] * 4);
+        }
+    };
+    auto lstore = [&](int slot, int buf) {
+        float* S = smem + buf * STAGE;
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+            if (lval[i]) *reinterpret_cast<int4v*>(&S[lrow[i] * ROWE + lcc[i] * 4]) = st[slot][i];
+    };
+
+    gload(0, 0);
+    if (NBLK > 1) gload(1, 1);
+    float4v u[NK8];
+    {
+        const float* Up = Uf + ((((size_t)p * (Kp / 32) + wave) * NK8) * 64 + lane) * 4;
+#pragma unroll
+        for (int j = 0; j < NK8; j++)
+            u[j] = *reinterpret_cast<const float4v*>(Up + (size_t)j * 64 * 4);
+    }
+    lstore(0, 0);
+    if (NBLK > 1) lstore(1, 1);
+    __syncthreads();
+
+    // rows past the last tile get an offset outside the buffer and are dropped
+    const size_t m_bytes = (size_t)T * Kp * sizeof(float);
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(M + (size_t)p * Tp * Kp, m_bytes);
+    const unsigned m_rowb = (unsigned)Kp * 4u;
+    constexpr int PPR = CW / 4;                  // 16-byte pieces per row
+    auto send_rows = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int piece = tid + i * NT;
+            const int r = piece / PPR;
+            const int cc = piece - r * PPR;
+            const int4v v = *reinterpret_cast<const int4v*>(obuf + r * OROW + cc * 4);
+            const unsigned row = (unsigned)((blk0 + s) * 32 + r);
+            __builtin_amdgcn_raw_buffer_store_b128(v, rM, row * m_rowb + (unsigned)cc * 16u, 0,
+                                                   kStoreThrough);
+        }
+    };
+
+    const int frag = jrow * ROWE + hh * 4;
+    // NBLK bounds the steps; a work-group leaves after its own nreal (the same for all its
+    // threads): a step costs 128 matrix instructions here, so the blocks of a position are
+    // split evenly over the work-groups (gemm_stream_split) and none runs an idle step.
+    int last = 0;
+#pragma unroll
+    for (int s = 0; s < NBLK; s++) {
+        if (s >= nreal) break;
+        last = s;
+        if (s + D < NBLK) gload(s % D, s + D);
+        if (s > 0) send_rows(s - 1);
+        // the requests above stay above: left to itself the scheduler moves them down to the
+        // LDS stores that consume them, and a step then ends in a wait for memory
+        __builtin_amdgcn_sched_barrier(0);
+        const float* S = smem + (s % 3) * STAGE + frag;
+        float16v acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+        // two fragment registers in turn: the read that refills one is issued behind the
+        // four instructions that used it and has the other's four to arrive in
+        static_assert(NK8 % 2 == 0, "fragments are read in pairs");
+        float4v fa = *reinterpret_cast<const float4v*>(S);
+        float4v fb = *reinterpret_cast<const float4v*>(S + 8);
+#pragma unroll
+        for (int j = 0; j < NK8; j += 2) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j].x, fa.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j].y, fa.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j].z, fa.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j].w, fa.w, acc, 0, 0, 0);
+            if (j + 2 < NK8) fa = *reinterpret_cast<const float4v*>(S + (j + 2) * 8);
+            __builtin_amdgcn_sched_barrier(0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j + 1].x, fb.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j + 1].y, fb.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j + 1].z, fb.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(u[j + 1].w, fb.w, acc, 0, 0, 0);
+            if (j + 3 < NK8) fb = *reinterpret_cast<const float4v*>(S + (j + 3) * 8);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (s + 2 < NBLK) lstore((s + 2) % D, (s + 2) % 3);
+        __syncthreads();   // every wavefront has sent the rows of the block before
+        float* O = obuf + jrow * OROW + wave * 32 + hh * 8;
+        *reinterpret_cast<float4v*>(O) = float4v{acc[0], acc[1], acc[2], acc[3]};
+        *reinterpret_cast<float4v*>(O + 4) = float4v{acc[4], acc[5], acc[6], acc[7]};
+        *reinterpret_cast<float4v*>(O + 16) = float4v{acc[8], acc[9], acc[10], acc[11]};
+        *reinterpret_cast<float4v*>(O + 20) = float4v{acc[12], acc[13], acc[14], acc[15]};
+        __syncthreads();
+    }
+    send_rows(last);
+}
+
 // Fragment-order copy of one layer's filters for wino_gemm_stream_k, built on the host:
 // src is the reference layout [36][C][F] (F fastest), dst [36][Kp/32][Cp/16][64][8].
 void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, half_t* dst) {
@@ -1631,9 +1799,26 @@ void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, half_t
                 }
 }
 
-// Blocks per work-group for T tile rows: the fewest (a power of two up to kStreamBlocks)
-// with which one round of work-groups covers the 256 compute units, so that a batch of 8
-// boards runs one block per work-group, 64 boards eight and 128 boards sixteen.
+// The same for wino_gemm_stream32_k: dst [36][Kp/32][Cp/8][64][4] floats.
+void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, float* dst) {
+    const int nk8 = Cp / 8, nwb = Kp / 32;
+    for (int p = 0; p < kPos; p++)
+        for (int wb = 0; wb < nwb; wb++)
+            for (int j = 0; j < nk8; j++)
+                for (int l = 0; l < 64; l++) {
+                    const int k = 32 * wb + gemm_stream_channel(l & 31);
+                    for (int e = 0; e < 4; e++) {
+                        const int c = 8 * j + 4 * (l >> 5) + e;
+                        float v = 0.0f;
+                        if (c < C && k < F) v = src[((size_t)p * C + c) * F + k];
+                        dst[((((size_t)p * nwb + wb) * nk8 + j) * 64 + l) * 4 + e] = v;
+                    }
+                }
+}
+
+// Blocks per work-group for T tile rows in the fp16 kernel: the fewest (a power of two up
+// to kStreamBlocks) with which one round of work-groups covers the 256 compute units, so
+// that a batch of 8 boards runs one block per work-group, 64 boards eight and 128 sixteen.
 static int gemm_stream_blocks(int T, int Kp) {
     const int nblk = (T + 31) / 32;
     const int per_pos = 256 / (kPos * ((Kp + 255) / 256));   // work-groups per position in one round
@@ -1642,13 +1827,36 @@ static int gemm_stream_blocks(int T, int Kp) {
     return nb;
 }
 
-// Whether launch_gemm takes the streaming kernel for this shape (the caller then has to
-// hold the fragment-order filters): fp16 nets of 128, 192 and 256 filters (one column tile
-// of Kp / 32 wavefronts), input layer (64 padded planes) and tower layers, any batch.
-// (At 64 filters the tiled kernel is as fast: measured 3.0 against 3.5 us at 4 boards, 3.5
-// against 3.5 at 33.)
-bool gemm_stream_shape(int T, int Cp, int Kp) {
-    return T >= 1 && (Kp == 128 || Kp == 192 || Kp == 256) && (Cp == 64 || Cp == Kp);
+// The fp32 kernel's split of a position's 32-row blocks over work-groups: as many work-groups per
+// position as one round over the 256 compute units allows (7 at one column tile: 252
+// work-groups), fewer when there are fewer blocks, more when a work-group would otherwise
+// get more than kStreamBlocks.  A work-group takes floor or ceil of blocks / chunks and
+// leaves after its own; the kernel is instantiated for the next power of two.
+struct StreamSplit { int chunks, nb; };
+static StreamSplit gemm_stream_split(int T, int Kp) {
+    const int nblk = (T + 31) / 32;
+    const int per_pos = 256 / (kPos * ((Kp + 255) / 256));
+    int chunks = nblk < per_pos ? nblk : per_pos;
+    const int least = (nblk + kStreamBlocks - 1) / kStreamBlocks;
+    if (chunks < least) chunks = least;
+    const int most = (nblk + chunks - 1) / chunks;   // blocks of the largest share
+    int nb = 1;
+    while (nb < most) nb *= 2;
+    return {chunks, nb};
+}
+
+// Whether launch_gemm takes a streaming kernel for this shape (the caller then has to hold
+// the fragment-order filters): nets of 128, 192 and 256 filters (one column tile of Kp / 32
+// wavefronts), input layer (64 padded planes) and tower layers.  fp16: any batch (at 64
+// filters the tiled kernel is as fast: 3.0 against 3.5 us at 4 boards, 3.5 against 3.5 at
+// 33).  fp32: any batch at 128 and 256 filters (64 boards, 256 filters: 88 -> 84 us per
+// launch, 48 boards 78 -> 60, 8 boards 22 -> 13; 128 filters: 27 -> 24 at 64 boards); at 192
+// filters six wavefronts sit unevenly on four SIMDs and the tiled kernel is ahead from 24
+// boards (26.4 against 28.2 us; 16 boards 20.0 against 17.0), so tower layers stream up to 16.
+bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes) {
+    if (T < 1 || !(Kp == 128 || Kp == 192 || Kp == 256) || !(Cp == 64 || Cp == Kp)) return false;
+    if (elem_bytes == 4 && Kp == 192 && Cp == 192 && T > 16 * 25) return false;
+    return true;
 }
 
 template <int NKC, int NW>
@@ -1687,6 +1895,41 @@ static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int
         case 256: launch_gemm_stream_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
         case 192: launch_gemm_stream_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
         default: launch_gemm_stream_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
+    }
+}
+
+template <int NK8, int NW>
+static void launch_gemm_stream32_nk(const float* V, const float* Uf, float* M, int T, int Tp,
+                                    int Kp, hipStream_t s, LaunchTimer* t) {
+    const int nblk = (T + 31) / 32;
+    const StreamSplit sp = gemm_stream_split(T, Kp);
+    const int nb = sp.nb, chunks = sp.chunks;
+    const int seg = (kPos * chunks + 7) / 8;
+    const dim3 grid(8 * seg), block(64 * NW);
+    switch (nb) {
+        case 1: launch(wino_gemm_stream32_k<NK8, 1, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, seg); break;
+        case 2: launch(wino_gemm_stream32_k<NK8, 2, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, seg); break;
+        case 4: launch(wino_gemm_stream32_k<NK8, 4, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, seg); break;
+        case 8: launch(wino_gemm_stream32_k<NK8, 8, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, seg); break;
+        default: launch(wino_gemm_stream32_k<NK8, 16, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, seg); break;
+    }
+}
+
+template <int NW>
+static void launch_gemm_stream32_nw(const float* V, const float* Uf, float* M, int T, int Tp,
+                                    int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
+    if (Cp == 64)
+        launch_gemm_stream32_nk<8, NW>(V, Uf, M, T, Tp, Kp, s, t);
+    else
+        launch_gemm_stream32_nk<4 * NW, NW>(V, Uf, M, T, Tp, Kp, s, t);
+}
+
+static void launch_gemm_stream(const float* V, const float* Uf, float* M, int T, int Tp, int Cp,
+                               int Kp, hipStream_t s, LaunchTimer* t) {
+    switch (Kp) {
+        case 256: launch_gemm_stream32_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
+        case 192: launch_gemm_stream32_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
+        default: launch_gemm_stream32_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
     }
 }
 
@@ -1729,11 +1972,9 @@ void launch_gemm(const P* V, const P* U, const P* Uf, P* M, int T, int Tp, int C
                  hipStream_t s, LaunchTimer* t) {
     constexpr int BK = 128 / (int)sizeof(P);
     const int nk = Cp / BK;
-    if constexpr (sizeof(P) == 2) {
-        if (Uf != nullptr && gemm_stream_shape(T, Cp, Kp)) {
-            launch_gemm_stream(V, Uf, M, T, Tp, Cp, Kp, s, t);
-            return;
-        }
+    if (Uf != nullptr && gemm_stream_shape(T, Cp, Kp, (int)sizeof(P))) {
+        launch_gemm_stream(V, Uf, M, T, Tp, Cp, Kp, s, t);
+        return;
     }
     // The 256 x 256 tile pays off once its tiles can occupy most of the 256 compute units
     // (measured at 256 filters: from 6 row tiles = 216 work-groups, batch 52; with 5 = 180 the

@@ -507,17 +507,20 @@ def test_error_behaviour_on_device(pkg, netgen):
         p.initialize(64)
 
 
+@pytest.mark.parametrize("precision", [1, 0])
 @pytest.mark.parametrize("filters,batch", [(128, 1), (128, 9), (128, 30), (128, 52), (128, 72),
-                                           (192, 2), (192, 17), (192, 40), (192, 64)])
-def test_fp16_streaming_gemm_at_narrower_widths(pkg, netgen, orc, filters, batch):
-    """fp16 nets of 128 and 192 filters run the streaming GEMM with 4 and 6 wavefronts per
-    work-group (256 filters: 8); the batches take every number of blocks per work-group
-    (1, 2, 4, 8, 16), with tile counts that are not multiples of the 32-row block."""
-    print("case: fp16 streaming width %d b%d" % (filters, batch), flush=True)
-    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, filters, 5100 + filters, pkg.FP16,
+                                           (192, 2), (192, 16), (192, 17), (192, 40), (192, 64)])
+def test_streaming_gemm_at_narrower_widths(pkg, netgen, orc, filters, batch, precision):
+    """Nets of 128 and 192 filters run the streaming GEMM with 4 and 6 wavefronts per
+    work-group (256 filters: 8), in fp16 at every batch and in fp32 at every batch for 128
+    filters and up to 16 boards for 192 (the tiled kernel beyond: 17, 40 and 64 boards check
+    that hand-over).  The batches take every number of blocks per work-group (1, 2, 4, 8, 16),
+    with tile counts that are not multiples of the 32-row block."""
+    print("case: streaming width %d b%d precision=%d" % (filters, batch, precision), flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, filters, 5100 + filters, precision,
                                        batch)
     x = netgen.synthetic_inputs(batch, seed=filters + batch)
-    check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16,
+    check_outputs(pkg, orc, pipe, ref, h_ref, x, precision,
                   idx=sorted({0, batch // 2, batch - 1}))
     pipe.close()
 
