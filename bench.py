@@ -207,6 +207,15 @@ def netbench_workload(args, pkg, netgen):
     print(json.dumps(out))
 
 
+def gemm_kernel_name(fp16, Fp, B):
+    """The GEMM kernel the library launches for this precision, padded width and batch."""
+    if fp16 and Fp in (128, 192, 256):
+        return "wino_gemm_stream_k"
+    if not fp16 and (Fp in (128, 256) or (Fp == 192 and B <= 16)):
+        return "wino_gemm_stream32_k"
+    return "wino_gemm_k / wino_gemm_big_k family"
+
+
 def measure_forward(pkg, netgen, torch, blocks, F, precision, B, steps, warmup, lanes_arg,
                     profile_reps, host_buffers=False, blocks_of_k=0):
     """One network on the device: evaluations/s of `steps` forwards of B device-resident
@@ -328,8 +337,7 @@ def measure_forward(pkg, netgen, torch, blocks, F, precision, B, steps, warmup, 
     gemm_rate = gf / (ms[pkg.K_GEMM] * 1e-3)
     Fp = (F + 63) // 64 * 64
     roofline = {
-        "kernel": ("wino_gemm_stream_k" if (prec == pkg.FP16 and Fp == 256) else
-                   "wino_gemm_k / wino_gemm_big_k family") + " (36-way batched Winograd GEMM)",
+        "kernel": gemm_kernel_name(prec == pkg.FP16, Fp, B) + " (36-way batched Winograd GEMM)",
         "bound": "mfma", "achieved": gemm_rate / 1e12, "peak": peak / 1e12, "unit": "TFLOP/s",
         "frac": gemm_rate / peak,
         "traffic": measured_gemm_traffic(blocks, F, precision, B),
