@@ -211,7 +211,7 @@ def gemm_kernel_name(fp16, Fp, B):
     """The GEMM kernel the library launches for this precision, padded width and batch."""
     if fp16 and Fp in (128, 192, 256):
         return "wino_gemm_stream_k"
-    if not fp16 and (Fp in (128, 256) or (Fp == 192 and B <= 16)):
+    if not fp16 and Fp in (128, 256):
         return "wino_gemm_stream32_k"
     return "wino_gemm_k / wino_gemm_big_k family"
 

@@ -1846,17 +1846,17 @@ static StreamSplit gemm_stream_split(int T, int Kp) {
 }
 
 // Whether launch_gemm takes a streaming kernel for this shape (the caller then has to hold
-// the fragment-order filters): nets of 128, 192 and 256 filters (one column tile of Kp / 32
-// wavefronts), input layer (64 padded planes) and tower layers.  fp16: any batch (at 64
-// filters the tiled kernel is as fast: 3.0 against 3.5 us at 4 boards, 3.5 against 3.5 at
-// 33).  fp32: any batch at 128 and 256 filters (64 boards, 256 filters: 88 -> 84 us per
-// launch, 48 boards 78 -> 60, 8 boards 22 -> 13; 128 filters: 27 -> 24 at 64 boards); at 192
-// filters six wavefronts sit unevenly on four SIMDs and the tiled kernel is ahead from 24
-// boards (26.4 against 28.2 us; 16 boards 20.0 against 17.0), so tower layers stream up to 16.
+// the fragment-order filters): input layer (64 padded planes) and tower layers, any batch, of
+// fp16 nets of 128, 192 and 256 filters (one column tile of Kp / 32 wavefronts; at 64 filters
+// the tiled kernel is as fast: 3.0 against 3.5 us at 4 boards, 3.5 against 3.5 at 33) and of
+// fp32 nets of 128 and 256 filters (64 boards, 256 filters: 88 -> 79-83 us per launch, 48
+// boards 78 -> 58, 8 boards 22 -> 13; 128 filters: 27 -> 23 at 64 boards).  fp32 at 192 filters
+// stays with the tiled kernel: six wavefronts sit unevenly on four SIMDs and it is ahead from
+// 24 boards (26.4 against 28.2 us; 16 boards 20.0 against 17.0), and one kernel family per
+// network keeps a position's result independent of the batch it is evaluated in.
 bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes) {
-    if (T < 1 || !(Kp == 128 || Kp == 192 || Kp == 256) || !(Cp == 64 || Cp == Kp)) return false;
-    if (elem_bytes == 4 && Kp == 192 && Cp == 192 && T > 16 * 25) return false;
-    return true;
+    if (T < 1 || !(Cp == 64 || Cp == Kp)) return false;
+    return Kp == 128 || Kp == 256 || (Kp == 192 && elem_bytes == 2);
 }
 
 template <int NKC, int NW>
@@ -1926,11 +1926,10 @@ static void launch_gemm_stream32_nw(const float* V, const float* Uf, float* M, i
 
 static void launch_gemm_stream(const float* V, const float* Uf, float* M, int T, int Tp, int Cp,
                                int Kp, hipStream_t s, LaunchTimer* t) {
-    switch (Kp) {
-        case 256: launch_gemm_stream32_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
-        case 192: launch_gemm_stream32_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
-        default: launch_gemm_stream32_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
-    }
+    if (Kp == 256)
+        launch_gemm_stream32_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t);
+    else
+        launch_gemm_stream32_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t);
 }
 
 template <typename P, int NK>

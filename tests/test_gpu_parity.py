@@ -268,21 +268,24 @@ def test_handle_created_from_a_weights_file(pkg, netgen, orc, tmp_path):
 
 
 @pytest.mark.parametrize("precision", [0, 1])
-def test_batch_composition_does_not_change_results(pkg, netgen, orc, precision):
+@pytest.mark.parametrize("filters,maxb", [(64, 8), (128, 40), (192, 40), (256, 40)])
+def test_batch_composition_does_not_change_results(pkg, netgen, orc, precision, filters, maxb):
     """A position evaluated alone, in a partial batch and in a full batch gives
-    bit-identical planes (rows of the GEMM are independent)."""
-    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 2, 64, 77, precision, 8)
-    x = netgen.synthetic_inputs(8, seed=5)
-    pol8, val8 = pipe.forward_batch(x)
-    pol3, val3 = pipe.forward_batch(x[2:5])
-    pol1, val1 = pipe.forward_batch(x[4:5])
-    assert np.array_equal(pol8[2:5], pol3) and np.array_equal(val8[2:5], val3)
-    assert np.array_equal(pol8[4:5], pol1) and np.array_equal(val8[4:5], val1)
+    bit-identical planes: rows of the GEMM are independent, and a network's layers run one
+    kernel family at every batch (whatever the tile shapes, blocks per work-group or channel
+    groups the batch selects, a value is summed in the same order)."""
+    print("case: batch composition %d filters precision=%d" % (filters, precision), flush=True)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 2, filters, 77, precision, maxb)
+    x = netgen.synthetic_inputs(maxb, seed=5)
+    pol_all, val_all = pipe.forward_batch(x)
+    for lo, hi in ((2, 5), (4, 5), (0, min(17, maxb)), (1, min(34, maxb)), (0, 1)):
+        pol, val = pipe.forward_batch(x[lo:hi])
+        assert np.array_equal(pol_all[lo:hi], pol) and np.array_equal(val_all[lo:hi], val), (lo, hi)
     # a larger batch after a smaller one (stale rows in the padded tile range)
-    pol8b, val8b = pipe.forward_batch(x)
-    assert np.array_equal(pol8, pol8b) and np.array_equal(val8, val8b)
+    pol_b, val_b = pipe.forward_batch(x)
+    assert np.array_equal(pol_all, pol_b) and np.array_equal(val_all, val_b)
     with pytest.raises(ValueError):
-        pipe.forward_batch(np.zeros((9, 18, 361), np.float32))
+        pipe.forward_batch(np.zeros((maxb + 1, 18, 361), np.float32))
     pipe.close()
 
 
@@ -512,10 +515,9 @@ def test_error_behaviour_on_device(pkg, netgen):
                                            (192, 2), (192, 16), (192, 17), (192, 40), (192, 64)])
 def test_streaming_gemm_at_narrower_widths(pkg, netgen, orc, filters, batch, precision):
     """Nets of 128 and 192 filters run the streaming GEMM with 4 and 6 wavefronts per
-    work-group (256 filters: 8), in fp16 at every batch and in fp32 at every batch for 128
-    filters and up to 16 boards for 192 (the tiled kernel beyond: 17, 40 and 64 boards check
-    that hand-over).  The batches take every number of blocks per work-group (1, 2, 4, 8, 16),
-    with tile counts that are not multiples of the 32-row block."""
+    work-group (256 filters: 8); in fp32 only the 128-filter ones do, 192 filters stay on the
+    tiled kernels there.  The batches take every number of blocks per work-group (1, 2, 4, 8,
+    16), with tile counts that are not multiples of the 32-row block."""
     print("case: streaming width %d b%d precision=%d" % (filters, batch, precision), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, filters, 5100 + filters, precision,
                                        batch)
