@@ -228,29 +228,42 @@ public:
         HIP_CHECK(hipSetDevice(m_device));
         const int F = m_filters;
         m_layers.resize(n_layers);
-        std::vector<P> tmp;
+        // Filters are laid out on the host in fp32; an fp16 net converts them on the device.
+        std::vector<float> tmp;
+        DevBuf<float> stage;
+        auto upload = [&](DevBuf<P>& d) {
+            d.alloc(tmp.size());
+            if constexpr (sizeof(P) == 4) {
+                HIP_CHECK(hipMemcpy(d.p, tmp.data(), tmp.size() * sizeof(float),
+                                    hipMemcpyHostToDevice));
+            } else {
+                if (stage.count < tmp.size()) stage.alloc(tmp.size());
+                HIP_CHECK(hipMemcpy(stage.p, tmp.data(), tmp.size() * sizeof(float),
+                                    hipMemcpyHostToDevice));
+                convert_filters(stage.p, d.p, tmp.size(), ln.stream);
+                HIP_CHECK(hipGetLastError());
+                HIP_CHECK(hipStreamSynchronize(ln.stream));
+            }
+        };
         for (int l = 0; l < n_layers; l++) {
             Layer& L = m_layers[l];
             L.C = l == 0 ? kInPlanes : F;
             L.Cp = l == 0 ? m_C0p : m_Fp;
             // reference layout [36][C][F] (F fastest)  ->  [36][Fp][Cp] (C fastest),
             // zero padded (the role of zeropad_U, reference src/OpenCLScheduler.cpp:60-82)
-            tmp.assign((size_t)kPos * m_Fp * L.Cp, (P)0.0f);
+            tmp.assign((size_t)kPos * m_Fp * L.Cp, 0.0f);
             for (int p = 0; p < kPos; p++)
                 for (int c = 0; c < L.C; c++) {
                     const float* src = U[l] + ((size_t)p * L.C + c) * F;
                     for (int k = 0; k < F; k++)
-                        tmp[((size_t)p * m_Fp + k) * L.Cp + c] = (P)src[k];
+                        tmp[((size_t)p * m_Fp + k) * L.Cp + c] = src[k];
                 }
-            L.U.alloc(tmp.size());
-            HIP_CHECK(hipMemcpy(L.U.p, tmp.data(), tmp.size() * sizeof(P), hipMemcpyHostToDevice));
+            upload(L.U);
             // Second copy in the fragment order of the streaming GEMM, where some batch of
             // this handle can take that kernel (the smallest does if any).
             if (gemm_stream_shape(kTilesPerBoard, L.Cp, m_Fp, (int)sizeof(P))) {
-                build_stream_filters(U[l], L.C, F, L.Cp, m_Fp, tmp.data());
-                L.Uf.alloc(tmp.size());
-                HIP_CHECK(hipMemcpy(L.Uf.p, tmp.data(), tmp.size() * sizeof(P),
-                                    hipMemcpyHostToDevice));
+                build_stream_filters(U[l], L.C, F, L.Cp, m_Fp, (int)sizeof(P), tmp.data());
+                upload(L.Uf);
             }
             L.mean.assign(bn_mean[l], bn_mean[l] + F);
             L.scale.assign(bn_scale[l], bn_scale[l] + F);

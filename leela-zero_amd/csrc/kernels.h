@@ -59,10 +59,12 @@ template <typename P>
 void launch_gemm(const P* V, const P* U, const P* Uf, P* M, int T, int Tp, int Cp, int Kp,
                  hipStream_t s, LaunchTimer* t);
 bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes);
-// src [36][C][F] fp32 (F fastest) -> dst [36][Kp/32][Cp/16][64][8] fp16, zero padded.
-void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, _Float16* dst);
-// ... -> dst [36][Kp/32][Cp/8][64][4] fp32 for the fp32 streaming kernel.
-void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, float* dst);
+// src [36][C][F] fp32 (F fastest) -> dst in the operand order of the streaming kernel for
+// elements of elem_bytes (2: [36][Kp/32][Cp/16][64][8], 4: [36][Kp/32][Cp/8][64][4]), values
+// in fp32, zero padded; convert_filters turns such an array into fp16 on the device.
+void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, int elem_bytes,
+                          float* dst);
+void convert_filters(const float* src, _Float16* dst, size_t n, hipStream_t s);
 
 // M [36][Tp][Kp] -> out [n][361][Kp]:  max(0, scale*(A^T m A - mean) + rfac*res)
 template <typename P>

@@ -1781,39 +1781,43 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream32_k(const float* __r
     send_rows(last);
 }
 
-// Fragment-order copy of one layer's filters for wino_gemm_stream_k, built on the host:
-// src is the reference layout [36][C][F] (F fastest), dst [36][Kp/32][Cp/16][64][8].
-void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, half_t* dst) {
-    const int nkc = Cp / 16, nwb = Kp / 32;
+// Fragment-order copy of one layer's filters for the streaming kernels, built on the host
+// in fp32 (fp16 nets convert on the device, convert_filters): src is the reference layout
+// [36][C][F] (F fastest); dst is [36][Kp/32][Cp/16][64][8] for wino_gemm_stream_k
+// (elem_bytes 2) and [36][Kp/32][Cp/8][64][4] for wino_gemm_stream32_k (elem_bytes 4), zero
+// padded: a fragment is G consecutive input channels per lane, G = 16 / elem_bytes.
+void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, int elem_bytes,
+                          float* dst) {
+    const int G = 16 / elem_bytes;             // values per lane and fragment
+    const int nfr = Cp / (2 * G), nwb = Kp / 32;
     for (int p = 0; p < kPos; p++)
         for (int wb = 0; wb < nwb; wb++)
-            for (int kc = 0; kc < nkc; kc++)
+            for (int fr = 0; fr < nfr; fr++)
                 for (int l = 0; l < 64; l++) {
                     const int k = 32 * wb + gemm_stream_channel(l & 31);
-                    for (int e = 0; e < 8; e++) {
-                        const int c = 16 * kc + 8 * (l >> 5) + e;
+                    for (int e = 0; e < G; e++) {
+                        const int c = 2 * G * fr + G * (l >> 5) + e;
                         float v = 0.0f;
                         if (c < C && k < F) v = src[((size_t)p * C + c) * F + k];
-                        dst[((((size_t)p * nwb + wb) * nkc + kc) * 64 + l) * 8 + e] = (half_t)v;
+                        dst[((((size_t)p * nwb + wb) * nfr + fr) * 64 + l) * G + e] = v;
                     }
                 }
 }
 
-// The same for wino_gemm_stream32_k: dst [36][Kp/32][Cp/8][64][4] floats.
-void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, float* dst) {
-    const int nk8 = Cp / 8, nwb = Kp / 32;
-    for (int p = 0; p < kPos; p++)
-        for (int wb = 0; wb < nwb; wb++)
-            for (int j = 0; j < nk8; j++)
-                for (int l = 0; l < 64; l++) {
-                    const int k = 32 * wb + gemm_stream_channel(l & 31);
-                    for (int e = 0; e < 4; e++) {
-                        const int c = 8 * j + 4 * (l >> 5) + e;
-                        float v = 0.0f;
-                        if (c < C && k < F) v = src[((size_t)p * C + c) * F + k];
-                        dst[((((size_t)p * nwb + wb) * nk8 + j) * 64 + l) * 4 + e] = v;
-                    }
-                }
+// fp32 -> storage type on the device (round to nearest even, as a host cast would): the
+// filters of an fp16 net are laid out on the host in fp32 and converted here, which takes
+// the conversion of 2 x 191 M values out of push_weights' host time for a 40 x 256 net.
+__global__ __launch_bounds__(256) void convert_filters_k(const float* __restrict__ src,
+                                                         half_t* __restrict__ dst, size_t n) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+        dst[i] = (half_t)src[i];
+}
+
+void convert_filters(const float* src, half_t* dst, size_t n, hipStream_t s) {
+    const size_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(convert_filters_k, dim3((unsigned)(blocks < 2048 ? blocks : 2048)),
+                       dim3(256), 0, s, src, dst, n);
 }
 
 // Blocks per work-group for T tile rows in the fp16 kernel: the fewest (a power of two up
