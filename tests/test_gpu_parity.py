@@ -170,10 +170,12 @@ def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
     pipe.close()
 
 
-@pytest.mark.parametrize("blocks,filters,batch", [(20, 256, 32), (40, 256, 64)])
+@pytest.mark.parametrize("blocks,filters,batch", [(20, 256, 32), (40, 256, 64), (15, 192, 16),
+                                                  (10, 128, 24)])
 def test_forward_parity_deep_fp16(pkg, netgen, orc, blocks, filters, batch):
-    """The two large fp16 benchmark configurations (20x256 batch 32, 40x256 batch 64) at full
-    size: raw planes of every position of the batch against the oracle, head outputs of
+    """Deep fp16 towers: the two large fp16 benchmark configurations (20x256 batch 32, 40x256
+    batch 64) at full size, and 15x192 and 10x128 (the streaming GEMM with 6 and 4 wavefronts
+    under per-layer activation scales): raw planes of every position of the batch against the oracle, head outputs of
     three of them."""
     print("case: deep fp16 %dx%d b%d" % (blocks, filters, batch), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, blocks, filters, 2000 + blocks,
