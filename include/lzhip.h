@@ -125,7 +125,7 @@ int lzhip_forward_batch_device(lzhip_handle* h, int n, const void* d_in, void* d
  * :291).  Forwards enqueued on different lanes run side by side on the device, and
  * since a chain of dependent kernels leaves the device partly idle at every kernel
  * boundary, two batches on two lanes finish sooner than the same two on one.
- * A handle has two lanes, three when its max_batch is at most 32 (small batches leave
+ * A handle has two lanes, three when its max_batch is at most 48 (small batches leave
  * more of the device idle).  lzhip_forward_batch_device is lane 0; lzhip_forward_batch
  * and the request queue use one lane per batch in flight. */
 int lzhip_lanes(lzhip_handle* h);

@@ -127,8 +127,9 @@ public:
             throw std::runtime_error(std::string("device is ") + prop.gcnArchName +
                                      ", this library contains gfx950 code only");
         // Small batches leave more of the device idle at every kernel boundary: a third
-        // lane pays up to batch 32 (+10 %) and no longer at 64 (-2 %).
-        m_n_lanes = max_batch <= 32 ? 3 : 2;
+        // lane pays up to batch 48 (40x256 fp16: +1..30 % up to 32, +7 % at 40, +4 % at 48) and
+        // no longer from 52 (-2 % there, -6 % at 64).
+        m_n_lanes = max_batch <= 48 ? 3 : 2;
         if (const char* e = std::getenv("LZHIP_LANES")) {   // measurement knob: 1..3 lanes
             const int v = std::atoi(e);
             if (v >= 1 && v <= kLanes) m_n_lanes = v;

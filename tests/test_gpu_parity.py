@@ -361,7 +361,7 @@ def test_lanes_run_side_by_side_with_equal_results(pkg, netgen, orc):
     import torch
     print("case: lanes", flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 128, 81, pkg.FP16, 16)
-    assert pipe.lanes() == 3      # up to batch 32; two above
+    assert pipe.lanes() == 3      # up to batch 48; two above
     xa = netgen.synthetic_inputs(16, seed=21)
     xb = netgen.synthetic_inputs(11, seed=22)
     want_a = pipe.forward_batch(xa)
@@ -417,7 +417,7 @@ def test_lanes_run_side_by_side_with_equal_results(pkg, netgen, orc):
         rp, rv = ref.forward(xb[i])
         assert rel_l2(want_b[0][i], rp) <= 2e-2 and rel_l2(want_b[1][i], rv) <= 2e-2
     pipe.close()
-    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, 64, 82, pkg.FP16, 40)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 1, 64, 82, pkg.FP16, 52)
     assert pipe.lanes() == 2
     pipe.close()
 
