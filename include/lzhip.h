@@ -197,6 +197,10 @@ int lzhip_forward_eval(lzhip_handle* h, const float* in, float temperature, floa
 int lzhip_winograd_transform_f(const float* f, int outputs, int channels, float* U);
 /* process_bn_var (reference src/Network.cpp:151-157), in place. */
 int lzhip_process_bn_var(float* w, int n);
+/* Utils::ceilMultiple (reference src/Utils.cpp:208-215): a rounded up to a multiple of b
+ * (b > 0), the helper the reference pads its GEMM dimensions with (src/OpenCL.cpp:380-382).
+ * This library pads with it too: filters to 64 channels, tile rows to 256; b == 0 returns a. */
+size_t lzhip_ceil_multiple(size_t a, size_t b);
 
 /* ---- introspection used by the parity tests and the bench --------------- */
 

@@ -39,6 +39,7 @@ EXPORTS = [
     "lzhip_forward_batch_device_lane", "lzhip_forward_batch_device_noalloc", "lzhip_sync", "lzhip_stream",
     "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats", "lzhip_push_heads",
     "lzhip_evaluate_batch", "lzhip_forward_eval", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
+    "lzhip_ceil_multiple",
     "lzhip_debug_layer", "lzhip_get_act_scales", "lzhip_profile_forward", "lzhip_last_error",
     "lzhip_version",
 ]
@@ -156,6 +157,8 @@ def lib():
         L.lzhip_forward_eval.argtypes = [ctypes.c_void_p, _fp, ctypes.c_float, _fp, _fp]
         L.lzhip_winograd_transform_f.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp]
         L.lzhip_process_bn_var.argtypes = [_fp, ctypes.c_int]
+        L.lzhip_ceil_multiple.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
+        L.lzhip_ceil_multiple.restype = ctypes.c_size_t
         L.lzhip_debug_layer.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int] + [_fp] * 5
         L.lzhip_get_act_scales.argtypes = [ctypes.c_void_p, _fp, ctypes.c_int]
         L.lzhip_profile_forward.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 3 + \
@@ -207,6 +210,11 @@ def winograd_transform_f(f, outputs, channels):
     U = np.empty((36, channels, outputs), dtype=np.float32)
     _check(lib().lzhip_winograd_transform_f(_ptr(f), outputs, channels, _ptr(U)))
     return U
+
+
+def ceil_multiple(a, b):
+    """reference src/Utils.cpp:208-215: a rounded up to a multiple of b."""
+    return int(lib().lzhip_ceil_multiple(a, b))
 
 
 def process_bn_var(var):

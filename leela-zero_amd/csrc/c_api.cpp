@@ -312,6 +312,8 @@ int lzhip_process_bn_var(float* w, int n) {
     return LZHIP_OK;
 }
 
+size_t lzhip_ceil_multiple(size_t a, size_t b) { return lzhip::ceil_multiple(a, b); }
+
 int lzhip_debug_layer(lzhip_handle* h, int layer, int n, const float* act_in, const float* res,
                       float* V, float* M, float* Y) {
     if (!h || !act_in) return fail(LZHIP_EINVAL, "null argument");

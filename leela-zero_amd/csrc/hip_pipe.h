@@ -1,6 +1,7 @@
 // HIPPipe: the device executor behind the scheduler.  One instance owns the
 // weights, activation buffers and stream of one network on one GPU.
 #pragma once
+#include <cstddef>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -9,6 +10,14 @@
 #include "forward_pipe.h"
 
 namespace lzhip {
+
+// a rounded up to a multiple of b (Utils::ceilMultiple, reference src/Utils.cpp:208-215):
+// what the pipe pads its channel and tile counts with.
+inline size_t ceil_multiple(size_t a, size_t b) {
+    if (b == 0 || a % b == 0) return a;
+    return a + (b - a % b);
+}
+
 
 struct HeadWeightsHost {
     const float *bn_pol_mean, *bn_pol_scale, *ip_pol_w, *ip_pol_b;

@@ -29,7 +29,6 @@ typedef _Float16 half_t;
         }                                                                                   \
     } while (0)
 
-static inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 // Working memory of the entry point that allocates nothing (forward_device_static):
 // the buffers a lane otherwise gets from hipMalloc -- packed input planes, three
@@ -136,13 +135,13 @@ public:
         }
         // Every refusal comes before the first stream, event or allocation is made: a
         // constructor that throws runs no destructor.
-        m_Fp = round_up(filters, 64);
+        m_Fp = (int)ceil_multiple((size_t)filters, 64);
         if (!gemm_supports_channels<P>(m_Fp))
             throw std::invalid_argument(
                 "unsupported filter count: after rounding up to a multiple of 64, fp16 takes up "
                 "to 512 and 640, 768, 896, 1024; fp32 takes up to 512");
         m_C0p = 64;
-        m_Tp = round_up(max_batch * kTilesPerBoard, kTileRowPad);
+        m_Tp = (int)ceil_multiple((size_t)max_batch * kTilesPerBoard, kTileRowPad);
         // The transform kernels address V and M through 32-bit buffer offsets.
         if ((size_t)kPos * m_Tp * m_Fp * sizeof(P) >= ((size_t)1 << 31))
             throw std::invalid_argument(

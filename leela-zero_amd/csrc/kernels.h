@@ -6,7 +6,7 @@
 //   U    [36][Kp][Cp]        Winograd-domain filters, input channel fastest
 //   M    [36][Tp][Kp]        per-position GEMM results, output channel fastest
 // Cp, Kp are the channel counts padded to a multiple of 64, Tp the tile count
-// padded to a multiple of 128.  The contraction index (input channel) is the
+// padded to a multiple of 256.  The contraction index (input channel) is the
 // fastest-moving one of both GEMM operands, which is what the MFMA operand
 // registers want: each lane fetches 16 contiguous bytes of one row.
 #pragma once

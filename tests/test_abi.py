@@ -69,6 +69,19 @@ def test_bn_var_matches_oracle(pkg, orc):
     assert np.abs(pkg.process_bn_var(v) - orc.process_bn_var(v)).max() <= 1e-7
 
 
+def test_ceil_multiple_known_answers(pkg):
+    """The padding helper against the reference's own known answers
+    (UtilsTest.CeilMultiple, src/tests/utils_unittest.cpp:47-68)."""
+    cases = [(0, 1, 0), (0, 3, 0), (6, 1, 6), (23, 1, 23), (2, 2, 2), (4, 2, 4), (6, 2, 6),
+             (0, 3, 0), (3, 3, 3), (9, 3, 9), (3, 5, 5), (6, 5, 10), (9, 5, 10), (23, 5, 25),
+             (99, 100, 100)]
+    for a, b, want in cases:
+        assert pkg.ceil_multiple(a, b) == want, (a, b)
+    # the paddings the pipe applies with it: filters to 64 channels, tile rows to 256
+    assert pkg.ceil_multiple(18, 64) == 64 and pkg.ceil_multiple(192, 64) == 192
+    assert pkg.ceil_multiple(64 * 25, 256) == 1792
+
+
 def test_python_pipe_validates_call_order(pkg, netgen):
     pipe = pkg.HIPScheduler(pkg.FP32, 2)
     with pytest.raises(ValueError):
