@@ -181,6 +181,7 @@ private:
     std::deque<std::shared_ptr<Request>> m_queue;
     std::vector<std::thread> m_workers;
     bool m_collecting = false;  // one worker at a time assembles a batch
+    size_t m_wake_at = 1;       // queue length at which the collecting worker wants to be woken
     bool m_running = false;
     std::atomic<bool> m_draining{false};
     std::atomic<int> m_outstanding{0};  // callers currently inside forward()

@@ -166,6 +166,7 @@ int HIPScheduler::submit(const std::shared_ptr<Request>& req) {
     }
     req->packed = m_exec && m_exec->accepts_bits() && pack_planes(req->in, req->bits);
     m_outstanding++;
+    bool wake;
     {
         std::lock_guard<std::mutex> lk(m_mutex);
         if (!m_running) {
@@ -179,8 +180,12 @@ int HIPScheduler::submit(const std::shared_ptr<Request>& req) {
             return LZHIP_EHALT;
         }
         m_queue.push_back(req);
+        // The collecting worker sleeps until the queue has the length it waits for (or its
+        // grace period ends, or the device comes free: others notify it of those); waking
+        // every worker for every request in between only makes them queue up for this mutex.
+        wake = !m_collecting || m_queue.size() >= m_wake_at;
     }
-    m_cv.notify_all();  // the collecting worker and an idle one share this condition
+    if (wake) m_cv.notify_all();  // the collecting worker and an idle one share this condition
     int state;
     {
         std::unique_lock<std::mutex> lk(req->mu);
@@ -234,6 +239,7 @@ void HIPScheduler::worker() {
                 HIPScheduler* s;
                 ~Handover() {
                     s->m_collecting = false;
+                    s->m_wake_at = 1;
                     s->m_cv.notify_all();
                 }
             } handover{this};
@@ -243,6 +249,7 @@ void HIPScheduler::worker() {
             // Every executor slot taken: only a full batch is worth assembling ahead of
             // time; otherwise wait for a slot and decide then.
             if (m_exec_busy >= m_lanes) {
+                m_wake_at = (size_t)m_max_batch;
                 m_cv.wait(lk, [&] {
                     return !m_running || m_queue.empty() || m_exec_busy < m_lanes ||
                            (int)m_queue.size() >= m_max_batch;
@@ -258,6 +265,7 @@ void HIPScheduler::worker() {
             size_t target;
             if (pop <= m_max_batch) {
                 target = (size_t)std::max(1, pop);
+                m_wake_at = target;
                 if (cap_us > 0)
                     m_cv.wait(lk, [&] {
                         return !m_running || m_queue.empty() || m_inflight == 0 ||
@@ -267,6 +275,7 @@ void HIPScheduler::worker() {
             } else {
                 target = (size_t)std::max(1, std::min(m_max_batch, pop - m_inflight));
             }
+            m_wake_at = target;
             if (m_queue.size() < target && cap_us > 0) {
                 // system_clock: waits on it map to pthread_cond_timedwait, which thread
                 // sanitizers model; the grace period is far too short for clock steps
