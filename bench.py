@@ -502,7 +502,7 @@ def main():
     ap.add_argument("--profile-reps", type=int, default=5)
     ap.add_argument("--lanes", type=int, default=0,
                     help="forward workload: batches kept on the device side by side; 0 = as "
-                         "many as the handle has (2, or 3 up to batch 32)")
+                         "many as the handle has (2, or 3 up to batch 48)")
     ap.add_argument("--workload", choices=["forward", "search", "netbench"], default="forward",
                     help="forward: the headline metric; search: visits/s of a multi-threaded tree search; netbench: "
                          "the reference's Network::benchmark (threads x single-position requests)")

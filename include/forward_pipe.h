@@ -64,6 +64,19 @@ public:
 
 namespace lzhip {
 
+// Process-wide batch counters of every HIPScheduler: the place of the reference's global
+// batch_stats (reference src/OpenCLScheduler.h:43-49, counted at .cpp:367-373, printed
+// after every search by src/UCTSearch.cpp:855-860).  single_evals / batch_evals count
+// device batches of one position / of more, as there; positions and slots (batches x
+// max_batch) give the batch fill ratio.  Always counted (the reference: debug builds).
+struct batch_stats_t {
+    std::atomic<size_t> single_evals{0};
+    std::atomic<size_t> batch_evals{0};
+    std::atomic<size_t> positions{0};
+    std::atomic<size_t> slots{0};
+};
+extern batch_stats_t batch_stats;
+
 // What the scheduler drives: something that evaluates up to max_batch()
 // positions held in host memory and blocks until the results are back.
 // HIPPipe is the device implementation; the scheduler's unit tests plug in a

@@ -140,9 +140,14 @@ int lzhip_forward_batch_device_lane(lzhip_handle* h, int lane, int n, const void
  * the lane's allocated buffers.  The call launches kernels and nothing else.
  * Limits: 1 <= n <= LZHIP_NOALLOC_MAX_BATCH (and <= max_batch), networks of up to
  * LZHIP_NOALLOC_MAX_FILTERS filters; anything larger returns LZHIP_EINVAL with a
- * message.  All calls on one GPU share the array, from whatever handle: calls that
- * overlap on that GPU race (calls on one handle are ordered by its stream).
- * Returns without waiting; lzhip_sync waits. */
+ * message.  All calls on one GPU share the array, from whatever handle: the library
+ * orders them on the device (each call's kernels wait, through one event per GPU, for
+ * the kernels of the call enqueued before it), so calls from several handles or threads
+ * of one process do not overwrite each other's tiles; they do not run side by side
+ * either.  While the lane's stream is being captured into a graph that ordering is left
+ * out (no event is recorded into the capture): replays of such a graph that overlap
+ * with other users of the array race.  Two processes on one GPU each hold their own
+ * copy of the array.  Returns without waiting; lzhip_sync waits. */
 #define LZHIP_NOALLOC_MAX_BATCH 8
 #define LZHIP_NOALLOC_MAX_FILTERS 256
 int lzhip_forward_batch_device_noalloc(lzhip_handle* h, int n, const void* d_in, void* d_pol,
@@ -159,6 +164,11 @@ int lzhip_resume(lzhip_handle* h);
 
 int lzhip_get_stats(lzhip_handle* h, lzhip_stats* out);
 int lzhip_reset_stats(lzhip_handle* h);
+/* The reference's global batch_stats (src/OpenCLScheduler.h:43-49, printed after every
+ * search, src/UCTSearch.cpp:855-860), over every handle of the process since it started:
+ * out[0] = device batches of one position (single_evals), out[1] = batches of more
+ * (batch_evals), out[2] = positions in all batches, out[3] = batches x max_batch. */
+int lzhip_process_batch_stats(uint64_t out[4]);
 
 /* ---- heads computed on the device (reference computes them on the host,
  * src/Network.cpp:833-851) ------------------------------------------------ */

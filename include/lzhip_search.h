@@ -51,7 +51,9 @@ typedef struct lzhip_search_config {
     float puct;        /* 0.5                                                      */
     float logpuct;     /* 0.015                                                    */
     float logconst;    /* 1.7                                                      */
-    float fpu_reduction; /* 0.25 (root uses the same value)                        */
+    float fpu_reduction; /* 0.25: first-play urgency reduction below the root      */
+    float fpu_root_reduction; /* at the root; 0.25 (reference cfg_fpu_root_reduction,
+                                 src/GTP.cpp:354, used at src/UCTNode.cpp:322-324)  */
     float softmax_temp;  /* 1.0                                                    */
     float komi;          /* 7.5                                                    */
     uint64_t seed;

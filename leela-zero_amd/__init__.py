@@ -37,7 +37,8 @@ EXPORTS = [
     "lzhip_create", "lzhip_create_from_file", "lzhip_destroy", "lzhip_push_weights", "lzhip_forward",
     "lzhip_forward_batch", "lzhip_forward_batch_device", "lzhip_lanes",
     "lzhip_forward_batch_device_lane", "lzhip_forward_batch_device_noalloc", "lzhip_sync", "lzhip_stream",
-    "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats", "lzhip_push_heads",
+    "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats",
+    "lzhip_process_batch_stats", "lzhip_push_heads",
     "lzhip_evaluate_batch", "lzhip_forward_eval", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
     "lzhip_ceil_multiple",
     "lzhip_debug_layer", "lzhip_get_act_scales", "lzhip_profile_forward", "lzhip_last_error",
@@ -51,6 +52,16 @@ SEARCH_EXPORTS = [
 ]
 
 BLACK, WHITE, EMPTY, PASS = 0, 1, 2, 361
+
+
+def process_batch_stats():
+    """The process-wide counters the engine prints after a search (reference
+    src/UCTSearch.cpp:855-860): batches of one position, batches of more, positions
+    evaluated, batch slots offered."""
+    out = (ctypes.c_uint64 * 4)()
+    _check(lib().lzhip_process_batch_stats(out))
+    return dict(single_evals=int(out[0]), batch_evals=int(out[1]), positions=int(out[2]),
+                slots=int(out[3]))
 
 
 class NetworkHaltException(Exception):
@@ -89,6 +100,7 @@ class SearchConfig(ctypes.Structure):
                 ("device_heads", ctypes.c_int),
                 ("puct", ctypes.c_float), ("logpuct", ctypes.c_float),
                 ("logconst", ctypes.c_float), ("fpu_reduction", ctypes.c_float),
+                ("fpu_root_reduction", ctypes.c_float),
                 ("softmax_temp", ctypes.c_float), ("komi", ctypes.c_float),
                 ("seed", ctypes.c_uint64)]
 
@@ -152,6 +164,7 @@ def lib():
         L.lzhip_resume.argtypes = [ctypes.c_void_p]
         L.lzhip_get_stats.argtypes = [ctypes.c_void_p, ctypes.POINTER(Stats)]
         L.lzhip_reset_stats.argtypes = [ctypes.c_void_p]
+        L.lzhip_process_batch_stats.argtypes = [ctypes.POINTER(ctypes.c_uint64)]
         L.lzhip_push_heads.argtypes = [ctypes.c_void_p] + [_fp] * 10
         L.lzhip_evaluate_batch.argtypes = [ctypes.c_void_p, ctypes.c_int, _fp, ctypes.c_float] + [_fp] * 5
         L.lzhip_forward_eval.argtypes = [ctypes.c_void_p, _fp, ctypes.c_float, _fp, _fp]

@@ -233,6 +233,15 @@ int lzhip_reset_stats(lzhip_handle* h) {
     GUARD_END
 }
 
+int lzhip_process_batch_stats(uint64_t out[4]) {
+    if (!out) return fail(LZHIP_EINVAL, "null argument");
+    out[0] = lzhip::batch_stats.single_evals.load();
+    out[1] = lzhip::batch_stats.batch_evals.load();
+    out[2] = lzhip::batch_stats.positions.load();
+    out[3] = lzhip::batch_stats.slots.load();
+    return LZHIP_OK;
+}
+
 int lzhip_push_heads(lzhip_handle* h, const float* bn_pol_mean, const float* bn_pol_scale,
                      const float* ip_pol_w, const float* ip_pol_b, const float* bn_val_mean,
                      const float* bn_val_scale, const float* ip1_val_w,
@@ -507,6 +516,7 @@ int lzhip_search_default_config(lzhip_search_config* cfg) {
     cfg->logpuct = 0.015f;
     cfg->logconst = 1.7f;
     cfg->fpu_reduction = 0.25f;
+    cfg->fpu_root_reduction = cfg->fpu_reduction;
     cfg->softmax_temp = 1.0f;
     cfg->komi = 7.5f;
     cfg->seed = 1;

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <condition_variable>
@@ -54,6 +55,13 @@ static __device__ __align__(256) unsigned char scratch[kStaticBytes];
 constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mu;
 static unsigned char* g_scratch_ptr[kMaxDevices] = {};
+// One event per device, recorded behind every forward that uses the device's array and
+// waited for by the next one, whichever handle and stream it comes from: forwards of
+// different handles on one GPU then follow one another on the device instead of
+// overwriting each other's tiles.  g_scratch_order_mu makes "wait, enqueue, record" one
+// step, so the order of the records is the order of the waits.
+static hipEvent_t g_scratch_event[kMaxDevices] = {};
+static std::mutex g_scratch_order_mu;
 
 // Device address of this device's copy of `scratch`; resolved once per device, with
 // that device current (called from the pipe's constructor, i.e. from lzhip_create).
@@ -65,6 +73,7 @@ static unsigned char* static_scratch(int device) {
         unsigned char* ptr = nullptr;
         HIP_CHECK(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
         if (!ptr) throw std::runtime_error("hipGetSymbolAddress returned a null address");
+        HIP_CHECK(hipEventCreateWithFlags(&g_scratch_event[device], hipEventDisableTiming));
         g_scratch_ptr[device] = ptr;
     }
     return g_scratch_ptr[device];
@@ -217,6 +226,9 @@ public:
     std::vector<float> act_scales() const override { return m_s; }
 
     // -------------------------------------------------------------------
+    // All or nothing: a failure anywhere below (an allocation, a copy, the calibration)
+    // leaves the handle as it was before the call -- no layers, forwards refused, and a
+    // later push_weights accepted.
     void push_weights(int n_layers, const float* const* U, const float* const* bn_mean,
                       const float* const* bn_scale, const float* pol_w,
                       const float* val_w) override {
@@ -224,8 +236,23 @@ public:
         std::lock_guard<std::mutex> lk(ln.mu);
         if (n_layers < 1 || (n_layers % 2) != 1)
             throw std::invalid_argument("n_layers must be 1 + 2*blocks");
-        if (!m_layers.empty()) throw std::invalid_argument("push_weights called twice");
+        if (m_ready || !m_layers.empty()) throw std::invalid_argument("push_weights called twice");
         HIP_CHECK(hipSetDevice(m_device));
+        try {
+            build_layers(n_layers, U, bn_mean, bn_scale, pol_w, val_w);
+        } catch (...) {
+            (void)hipStreamSynchronize(ln.stream);
+            m_layers.clear();
+            m_w3.release();
+            m_s.clear();
+            throw;
+        }
+        m_ready = true;
+    }
+
+    void build_layers(int n_layers, const float* const* U, const float* const* bn_mean,
+                      const float* const* bn_scale, const float* pol_w, const float* val_w) {
+        auto& ln = m_lane[0];
         const int F = m_filters;
         m_layers.resize(n_layers);
         // Filters are laid out on the host in fp32; an fp16 net converts them on the device.
@@ -249,21 +276,23 @@ public:
             Layer& L = m_layers[l];
             L.C = l == 0 ? kInPlanes : F;
             L.Cp = l == 0 ? m_C0p : m_Fp;
-            // reference layout [36][C][F] (F fastest)  ->  [36][Fp][Cp] (C fastest),
-            // zero padded (the role of zeropad_U, reference src/OpenCLScheduler.cpp:60-82)
             tmp.assign((size_t)kPos * m_Fp * L.Cp, 0.0f);
-            for (int p = 0; p < kPos; p++)
-                for (int c = 0; c < L.C; c++) {
-                    const float* src = U[l] + ((size_t)p * L.C + c) * F;
-                    for (int k = 0; k < F; k++)
-                        tmp[((size_t)p * m_Fp + k) * L.Cp + c] = src[k];
-                }
-            upload(L.U);
-            // Second copy in the fragment order of the streaming GEMM, where some batch of
-            // this handle can take that kernel (the smallest does if any).
+            // One copy of the filters, in the order the GEMM of this width and precision
+            // reads them.  Whether that is the streaming kernel does not depend on the
+            // batch, so a network holds either the fragment order or the row order, never both.
             if (gemm_stream_shape(kTilesPerBoard, L.Cp, m_Fp, (int)sizeof(P))) {
                 build_stream_filters(U[l], L.C, F, L.Cp, m_Fp, (int)sizeof(P), tmp.data());
                 upload(L.Uf);
+            } else {
+                // reference layout [36][C][F] (F fastest)  ->  [36][Fp][Cp] (C fastest),
+                // zero padded (the role of zeropad_U, reference src/OpenCLScheduler.cpp:60-82)
+                for (int p = 0; p < kPos; p++)
+                    for (int c = 0; c < L.C; c++) {
+                        const float* src = U[l] + ((size_t)p * L.C + c) * F;
+                        for (int k = 0; k < F; k++)
+                            tmp[((size_t)p * m_Fp + k) * L.Cp + c] = src[k];
+                    }
+                upload(L.U);
             }
             L.mean.assign(bn_mean[l], bn_mean[l] + F);
             L.scale.assign(bn_scale[l], bn_scale[l] + F);
@@ -299,14 +328,18 @@ public:
     // The same forward with every working buffer taken from the device's static
     // `scratch` array instead of the lane's allocations: kernel launches only, no
     // allocation of any kind.  Enqueued on lane 0's stream.  All calls on one GPU share
-    // the array (whatever the handle), so calls that overlap on that GPU race; calls on
-    // one handle are ordered by the stream.  Nothing in the array has to start at zero:
-    // every element a kernel reads for a real tile is written earlier in the same call
-    // (rows of V past the last tile feed only rows of M that no kernel reads).
+    // the array (whatever the handle): each waits on the device for the one enqueued
+    // before it (one event per device, see g_scratch_event), so calls from different
+    // handles or threads of this process run one after the other on the device.  While
+    // the stream is being captured into a graph no event is recorded or waited for (the
+    // captured launches are then ordered by the graph's own dependencies, and replays
+    // that overlap with other users of the array race).  Nothing in the array has to
+    // start at zero: every element a kernel reads for a real tile is written earlier in
+    // the same call (rows of V past the last tile feed only rows of M that no kernel reads).
     void forward_device_static(int n, const float* d_in, float* d_pol, float* d_val) override {
         Lane& ln = m_lane[0];
         std::lock_guard<std::mutex> lk(ln.mu);
-        if (m_layers.empty()) throw std::invalid_argument("push_weights has not been called");
+        if (!m_ready) throw std::invalid_argument("push_weights has not been called");
         if (n < 1 || n > kStaticMaxBatch || n > m_max_batch)
             throw std::invalid_argument(
                 "the no-allocation forward takes 1..8 positions (and at most max_batch): its "
@@ -326,8 +359,15 @@ public:
         for (int i = 0; i < 3; i++)
             w.act[i] = reinterpret_cast<P*>(base + 2 * kStaticTileBytes + kStaticAct0Bytes +
                                             (size_t)i * kStaticActBytes);
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        HIP_CHECK(hipStreamIsCapturing(ln.stream, &cap));
+        const bool ordered = cap == hipStreamCaptureStatusNone;
+        std::lock_guard<std::mutex> order(g_scratch_order_mu);
+        hipEvent_t ev = g_scratch_event[m_device];
+        if (ordered) HIP_CHECK(hipStreamWaitEvent(ln.stream, ev, 0));
         enqueue_forward(w, n, d_in, nullptr, d_pol, d_val, false);
         HIP_CHECK(hipGetLastError());
+        if (ordered) HIP_CHECK(hipEventRecord(ev, ln.stream));
     }
 
     void sync() override {
@@ -620,7 +660,7 @@ private:
     };
 
     void check_ready(int n) const {
-        if (m_layers.empty()) throw std::invalid_argument("push_weights has not been called");
+        if (!m_ready) throw std::invalid_argument("push_weights has not been called");
         if (n < 1 || n > m_max_batch) throw std::invalid_argument("batch size out of range");
     }
 
@@ -841,6 +881,7 @@ private:
     std::mutex m_slot_mu;
     std::condition_variable m_slot_cv;
     std::vector<Layer> m_layers;
+    std::atomic<bool> m_ready{false};   // set by a push_weights that ran to its end
     std::vector<float> m_s;  // activation scales, m_s[0] = input
     DevBuf<float> m_h[10], m_dpolicy, m_dlogits, m_dvalue, m_dwork;
     bool m_heads_ready = false;

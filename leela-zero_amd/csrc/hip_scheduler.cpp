@@ -19,6 +19,8 @@
 
 namespace lzhip {
 
+batch_stats_t batch_stats;
+
 static constexpr int kInSize = LZHIP_INPUT_SIZE;
 static constexpr int kPolSize = LZHIP_POL_SIZE;
 static constexpr int kValSize = LZHIP_VAL_SIZE;
@@ -346,6 +348,9 @@ void HIPScheduler::worker() {
         }
         m_cv.notify_all();  // a collector may be waiting for the device to come free
         m_batches++;
+        (n == 1 ? batch_stats.single_evals : batch_stats.batch_evals)++;
+        batch_stats.positions += (size_t)n;
+        batch_stats.slots += (size_t)m_max_batch;
         uint32_t seen = m_max_seen.load();
         while ((uint32_t)n > seen && !m_max_seen.compare_exchange_weak(seen, (uint32_t)n)) {}
         for (int i = 0; i < n; i++) {

@@ -290,13 +290,14 @@ float puct_eval_for(int tomove, double blackevals, int visits, int virtual_loss)
     return e;
 }
 
-PuctParent puct_parent(const lzhip_search_config& cfg, size_t children_visits,
+PuctParent puct_parent(const lzhip_search_config& cfg, bool is_root, size_t children_visits,
                        float visited_policy, float parent_eval_for_color) {
     PuctParent p;
     p.numerator = std::sqrt((double)children_visits *
                             std::log((double)cfg.logpuct * (double)children_visits +
                                      (double)cfg.logconst));
-    p.fpu_reduction = cfg.fpu_reduction * std::sqrt(visited_policy);
+    p.fpu_reduction =
+        (is_root ? cfg.fpu_root_reduction : cfg.fpu_reduction) * std::sqrt(visited_policy);
     p.fpu_eval = parent_eval_for_color - p.fpu_reduction;
     return p;
 }
@@ -464,7 +465,7 @@ bool UCTSearch::create_children(Node* node, const go::Position& pos, float& eval
     return true;
 }
 
-Child* UCTSearch::select_child(Node* node, int color, bool /*is_root*/) {
+Child* UCTSearch::select_child(Node* node, int color, bool is_root) {
     float total_visited_policy = 0.0f;
     size_t parentvisits = 0;
     for (int i = 0; i < node->n_children; i++) {
@@ -476,7 +477,7 @@ Child* UCTSearch::select_child(Node* node, int color, bool /*is_root*/) {
         if (v > 0) total_visited_policy += c.prior;
     }
     const PuctParent parent =
-        puct_parent(m_cfg, parentvisits, total_visited_policy, node->raw_eval(color, 0));
+        puct_parent(m_cfg, is_root, parentvisits, total_visited_policy, node->raw_eval(color, 0));
 
     Child* best = nullptr;
     double best_value = std::numeric_limits<double>::lowest();

@@ -153,13 +153,14 @@ struct Child;
 float puct_eval_for(int tomove, double blackevals, int visits, int virtual_loss);
 // What the parent contributes: the exploration numerator sqrt(N ln(logpuct N + logconst))
 // over the children's visits N, and the value given to children without visits, the
-// parent's own mean for the side to move less fpu_reduction * sqrt(priors of the visited).
+// parent's own mean for the side to move less fpu_reduction * sqrt(priors of the visited)
+// (fpu_root_reduction when the parent is the root, reference src/UCTNode.cpp:322-324).
 struct PuctParent {
     double numerator;
     float fpu_reduction;
     float fpu_eval;
 };
-PuctParent puct_parent(const lzhip_search_config& cfg, size_t children_visits,
+PuctParent puct_parent(const lzhip_search_config& cfg, bool is_root, size_t children_visits,
                        float visited_policy, float parent_eval_for_color);
 // Selection value of one child: its mean (fpu_eval without visits, -1 - fpu_reduction
 // while another thread expands it) + puct * prior * numerator / (1 + visits).

@@ -181,12 +181,25 @@ static void test_concurrent(int threads, int mb, int reps, int concurrency = 1) 
     HIPScheduler s{std::unique_ptr<BatchExecutor>(fe)};
     std::atomic<int> ok{0}, halted{0};
     std::vector<std::thread> th;
+    // the process-wide counters the engine prints after a search (no other scheduler is
+    // running during this test, so their growth is this scheduler's)
+    const size_t g_single = batch_stats.single_evals, g_batch = batch_stats.batch_evals,
+                 g_pos = batch_stats.positions, g_slots = batch_stats.slots;
     for (int t = 0; t < threads; t++)
         th.emplace_back([&, t] {
             for (int r = 0; r < reps; r++) one_call(s, (float)(t * 1000 + r), (float)(r - t), ok, halted);
         });
     for (auto& t : th) t.join();
     CHECK(ok == threads * reps && halted == 0);
+    {
+        const lzhip_stats st = s.stats();
+        const size_t singles = batch_stats.single_evals - g_single;
+        const size_t multis = batch_stats.batch_evals - g_batch;
+        CHECK(singles + multis == st.batches);
+        CHECK(batch_stats.positions - g_pos == st.requests);
+        CHECK(batch_stats.slots - g_slots == st.batch_slots);
+        if (threads == 1) CHECK(multis == 0 && singles == st.requests);
+    }
     CHECK(!fe->oversize);
     CHECK(fe->positions == threads * reps);
     const lzhip_stats st = s.stats();

@@ -147,6 +147,7 @@ static lzhip_search_config config(int threads, int visits, int moves) {
     c.logpuct = 0.015f;
     c.logconst = 1.7f;
     c.fpu_reduction = 0.25f;
+    c.fpu_root_reduction = 0.25f;
     c.softmax_temp = 1.0f;
     c.komi = 7.5f;
     c.seed = 7;
@@ -450,7 +451,7 @@ static void test_puct_arithmetic() {
     const double blackevals[4] = {3.30, 1.95, 0.0, 0.0};
     auto near = [](double a, double b) { return std::fabs(a - b) < 2e-6; };
     auto pick = [&](const lzhip_search_config& c, int color, const int* vloss, int expanding,
-                    double* values) {
+                    double* values, bool is_root = false) {
         size_t n = 0;
         float visited = 0.0f;
         for (int i = 0; i < 4; i++) {
@@ -458,7 +459,7 @@ static void test_puct_arithmetic() {
             if (visits[i] > 0) visited += prior[i];
         }
         const float parent_eval = puct_eval_for(color, 5.5, 10, 0);
-        const PuctParent par = puct_parent(c, n, visited, parent_eval);
+        const PuctParent par = puct_parent(c, is_root, n, visited, parent_eval);
         int best = -1;
         double best_value = -1e300;
         for (int i = 0; i < 4; i++) {
@@ -473,7 +474,7 @@ static void test_puct_arithmetic() {
     };
     double v[4];
     {
-        const PuctParent par = puct_parent(cfg, 9, 0.70f, 0.55f);
+        const PuctParent par = puct_parent(cfg, false, 9, 0.70f, 0.55f);
         CHECK(near(par.numerator, 2.337392) && near(par.fpu_reduction, 0.209165) &&
               near(par.fpu_eval, 0.340835));
     }
@@ -483,6 +484,13 @@ static void test_puct_arithmetic() {
     lzhip_search_config no_fpu = cfg;
     no_fpu.fpu_reduction = 0.0f;
     CHECK(pick(no_fpu, go::BLACK, nullptr, -1, v) == 2 && near(v[2], 0.783739));
+    // the root has a reduction of its own (reference src/UCTNode.cpp:322-324): with none at
+    // the root and 0.25 below it the same node picks child 2 as the root and child 1 elsewhere
+    lzhip_search_config root_cfg = cfg;
+    CHECK(root_cfg.fpu_root_reduction == 0.25f);
+    root_cfg.fpu_root_reduction = 0.0f;
+    CHECK(pick(root_cfg, go::BLACK, nullptr, -1, v, true) == 2 && near(v[2], 0.783739));
+    CHECK(pick(root_cfg, go::BLACK, nullptr, -1, v, false) == 1 && near(v[2], 0.574574));
     CHECK(pick(cfg, go::WHITE, nullptr, -1, v) == 0);
     CHECK(near(v[0], 0.516783) && near(v[1], 0.437652) && near(v[2], 0.474574) &&
           near(v[3], 0.357705));

@@ -56,6 +56,42 @@ def heads_f64(net, pol, val, temperature=1.0, eps=1e-5):
     return dict(policy=policy, logits=logits, value=np.tanh(o), winrate=(1 + np.tanh(o)) / 2, value_pre=o)
 
 
+def normalise_network(net, x, branch_rms=0.15):
+    """Gives a RawNetwork the batch-norm statistics a trained network has: every layer's
+    mean and variance are set from what its convolution puts out on the positions x
+    [n][18][361] (float32 direct convolutions), so that the normalised output has zero mean
+    and unit RMS -- and RMS `branch_rms` on the second convolution of each block, which
+    keeps the residual stream O(1) however deep the tower is.  The two head planes are
+    normalised the same way.  Returns net (modified in place)."""
+    import torch
+    import torch.nn.functional as F
+    n = x.shape[0]
+    a = torch.from_numpy(np.asarray(x, np.float32).reshape(n, 18, 19, 19))
+
+    def conv_bn(inp, l, rms):
+        y = F.conv2d(inp, torch.from_numpy(net.conv_w[l]), padding=1)
+        mean = y.mean(dim=(0, 2, 3))
+        var = y.var(dim=(0, 2, 3), unbiased=False) / (rms * rms)
+        net.bn_mean[l] = mean.numpy().astype(np.float32)
+        net.bn_var[l] = np.maximum(var.numpy(), 1e-6).astype(np.float32)
+        net.conv_b[l] = np.zeros(net.filters, np.float32)
+        s = 1.0 / torch.sqrt(torch.from_numpy(net.bn_var[l]) + 1e-5)
+        return s[None, :, None, None] * (y - torch.from_numpy(net.bn_mean[l])[None, :, None, None])
+
+    a = torch.relu(conv_bn(a, 0, 1.0))
+    for l in range(1, net.n_layers, 2):
+        t = torch.relu(conv_bn(a, l, 1.0))
+        a = torch.relu(conv_bn(t, l + 1, branch_rms) + a)
+    flat = a.reshape(n, net.filters, 361)
+    pol = torch.einsum("oc,ncp->nop", torch.from_numpy(net.pol_conv_w.reshape(2, -1)), flat)
+    val = torch.einsum("oc,ncp->nop", torch.from_numpy(net.val_conv_w.reshape(1, -1)), flat)
+    net.pol_bn_mean = pol.mean(dim=(0, 2)).numpy().astype(np.float32)
+    net.pol_bn_var = pol.var(dim=(0, 2), unbiased=False).numpy().astype(np.float32)
+    net.val_bn_mean = val.mean(dim=(0, 2)).numpy().astype(np.float32)
+    net.val_bn_var = val.var(dim=(0, 2), unbiased=False).numpy().astype(np.float32)
+    return net
+
+
 def rel_l2(a, b):
     a = np.asarray(a, np.float64).ravel()
     b = np.asarray(b, np.float64).ravel()

@@ -31,11 +31,12 @@ def test_library_exports_every_search_symbol(pkg):
         assert hasattr(L, name), name
     assert sorted(pkg.SEARCH_EXPORTS) == declared
     # struct sizes the ctypes mirror assumes
-    assert ctypes.sizeof(pkg.SearchConfig) == 64
+    assert ctypes.sizeof(pkg.SearchConfig) == 72
     assert ctypes.sizeof(pkg.CHeadWeights) == 80
     cfg = pkg.SearchConfig.default()
     assert (cfg.threads, cfg.visits, cfg.moves, cfg.virtual_loss) == (16, 1600, 20, 3)
     assert abs(cfg.puct - 0.5) < 1e-7 and abs(cfg.komi - 7.5) < 1e-7
+    assert cfg.fpu_reduction == 0.25 and cfg.fpu_root_reduction == 0.25 and cfg.seed == 1
     assert L.lzhip_selfplay(None, None, None, None, None, 0) == pkg.EINVAL
     assert L.lzhip_get_output(None, None, None, 1, 0, 0, ctypes.c_float(1.0), None, None) == pkg.EINVAL
 

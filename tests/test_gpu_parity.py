@@ -30,14 +30,19 @@ def make_pipes(pkg, netgen, orc, blocks, filters, seed, precision, max_batch):
 
 
 @pytest.mark.parametrize("precision", [0, 1])
-@pytest.mark.parametrize("filters", [8, 64, 192])
-def test_single_layer_stages(pkg, netgen, orc, precision, filters):
+@pytest.mark.parametrize("filters,n", [(8, 3), (64, 3), (192, 3), (128, 3), (128, 40), (256, 3),
+                                       (256, 40)])
+def test_single_layer_stages(pkg, netgen, orc, precision, filters, n):
     """V, M and Y of one convolution layer against the oracle's stages, for the input
-    layer (18 planes) and a residual-tower layer with a skip connection."""
-    print("case: single_layer precision=%d filters=%d" % (precision, filters), flush=True)
-    net, pipe, ref, _ = make_pipes(pkg, netgen, orc, 1, filters, 40 + filters, precision, 4)
+    layer (18 planes) and a residual-tower layer with a skip connection.  The M stage is
+    the check the reference's tuner makes of every GEMM it times, against a plain sgemm
+    (reference src/Tuner.cpp:262-301); 128 and 256 filters put the streaming GEMMs of both
+    storage types under it, at 3 boards (one 32-row block per work-group) and at 40 (several
+    blocks per work-group, a last block of 8 rows)."""
+    print("case: single_layer precision=%d filters=%d n=%d" % (precision, filters, n), flush=True)
+    net, pipe, ref, _ = make_pipes(pkg, netgen, orc, 1, filters, 40 + filters, precision,
+                                   max(4, n))
     rng = np.random.default_rng(filters)
-    n = 3
     tol = 1e-5 if precision == 0 else 4e-3
     # layer 0 on real input planes
     x = netgen.synthetic_inputs(n, seed=3)
@@ -46,9 +51,9 @@ def test_single_layer_stages(pkg, netgen, orc, precision, filters):
         Vr = orc.transform_in(x[i], 18)
         Mr = orc.sgemm(ref.U[0], Vr, 18, filters)
         Yr = orc.batchnorm(orc.transform_out(Mr, filters), ref.mean[0], ref.scale[0])
-        assert rel_l2(V[i], Vr) <= tol, "V layer0"
-        assert rel_l2(M[i], Mr) <= tol, "M layer0"
-        assert rel_l2(Y[i], Yr) <= tol, "Y layer0"
+        assert rel_l2(V[i], Vr) <= tol, ("V layer0", i)
+        assert rel_l2(M[i], Mr) <= tol, ("M layer0", i)
+        assert rel_l2(Y[i], Yr) <= tol, ("Y layer0", i)
     # layer 2 (second conv of the block) with a residual input
     a = np.abs(rng.standard_normal((n, filters, 361))).astype(np.float32)
     r = np.abs(rng.standard_normal((n, filters, 361))).astype(np.float32)
@@ -60,9 +65,9 @@ def test_single_layer_stages(pkg, netgen, orc, precision, filters):
         Vr = orc.transform_in(a[i], filters)
         Mr = orc.sgemm(ref.U[2], Vr, filters, filters)
         Yr = orc.batchnorm(orc.transform_out(Mr, filters), ref.mean[2], ref.scale[2], r[i])
-        assert rel_l2(V[i], Vr) <= tol, "V layer2"
-        assert rel_l2(M[i], Mr) <= tol, "M layer2"
-        assert rel_l2(Y[i], Yr) <= 2 * tol, "Y layer2"
+        assert rel_l2(V[i], Vr) <= tol, ("V layer2", i)
+        assert rel_l2(M[i], Mr) <= tol, ("M layer2", i)
+        assert rel_l2(Y[i], Yr) <= 2 * tol, ("Y layer2", i)
     pipe.close()
 
 
@@ -186,6 +191,76 @@ def test_forward_parity_deep_fp16(pkg, netgen, orc, blocks, filters, batch):
     assert np.all(s >= 1.0) and np.all(np.log2(s) == np.round(np.log2(s)))
     check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16, idx=[0, batch // 2, batch - 1],
                   all_raw=True)
+    pipe.close()
+
+
+def test_forward_parity_deep_fp16_with_plain_half_storage(pkg, netgen, orc):
+    """40x256 at batch 64 with batch-norm statistics that keep the activations O(1) through
+    all 40 blocks, as a trained network's do: the activation scales then come out as 1 for
+    every layer, i.e. plain half-precision storage as in the reference's half pipeline, the
+    heads are not saturated, and policy and value of all 64 positions are held to the fp16
+    tolerance where it bites (no position may take the ill-conditioned route here)."""
+    from helpers import normalise_network
+    print("case: deep fp16, normalised 40x256 b64", flush=True)
+    blocks, filters, batch = 40, 256, 64
+    net = normalise_network(netgen.make_network(blocks, filters, 2100),
+                            netgen.synthetic_inputs(4, seed=2101))
+    w, h = netgen.prepare(net)
+    w_ref, h_ref = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    ref = orc.OraclePipe()
+    ref.initialize(filters)
+    ref.push_weights(6, 18, filters, w_ref)
+    pipe = pkg.HIPScheduler(pkg.FP16, batch)
+    pipe.initialize(filters)
+    pipe.push_weights(6, 18, filters, w)
+    pipe.push_heads(h)
+    s = pipe.act_scales()
+    print("act scales: min %g max %g" % (s.min(), s.max()), flush=True)
+    assert np.all(s == 1.0), s
+    x = netgen.synthetic_inputs(batch, seed=2102)
+    worst = check_outputs(pkg, orc, pipe, ref, h_ref, x, pkg.FP16, all_raw=True)
+    assert worst["ill_conditioned"] == 0, worst
+    # not a saturated case: the mean policy maximum is far from one-hot, values spread
+    policy, value, _ = pipe.evaluate_batch(x)
+    print("policy max: mean %.3f; |value|: mean %.3f max %.3f"
+          % (policy.max(axis=1).mean(), np.abs(value).mean(), np.abs(value).max()), flush=True)
+    assert policy.max(axis=1).mean() < 0.9 and np.abs(value).mean() < 0.95
+    pipe.close()
+
+
+def test_failed_push_weights_leaves_the_handle_unchanged(pkg, netgen, orc):
+    """push_weights is all or nothing.  An fp16 push whose calibration cannot settle (a
+    layer with an infinite batch-norm scale: its activations are infinite at any scale) fails
+    after the filters of every layer went up; the handle must then refuse forwards exactly as
+    before any push, and accept a second push with good weights, whose results are right."""
+    print("case: failed push_weights", flush=True)
+    net = netgen.make_network(2, 64, 71)
+    w, h = netgen.prepare(net)
+    bad = pkg.ForwardPipeWeights()
+    bad.__dict__.update(w.__dict__)
+    bad.m_batchnorm_stddevs = [v.copy() for v in w.m_batchnorm_stddevs]
+    bad.m_batchnorm_stddevs[3][:] = np.inf
+    x = netgen.synthetic_inputs(3, seed=72)
+    pipe = pkg.HIPScheduler(pkg.FP16, 4)
+    pipe.initialize(64)
+    with pytest.raises(pkg.LzhipError):
+        pipe.push_weights(6, 18, 64, bad)
+    with pytest.raises(ValueError, match="push_weights has not been called"):
+        pipe.forward_batch(x)
+    import torch
+    d = torch.zeros(3, 18, 361, device="cuda")
+    o1, o2 = torch.zeros(3, 722, device="cuda"), torch.zeros(3, 361, device="cuda")
+    with pytest.raises(ValueError, match="push_weights has not been called"):
+        pipe.forward_batch_device_noalloc(3, d.data_ptr(), o1.data_ptr(), o2.data_ptr())
+    pipe.push_weights(6, 18, 64, w)            # accepted: the failed push left nothing behind
+    pol, val = pipe.forward_batch(x)
+    w_ref, _ = netgen.prepare(net, orc.winograd_transform_f, orc.process_bn_var)
+    ref = orc.OraclePipe()
+    ref.initialize(64)
+    ref.push_weights(6, 18, 64, w_ref)
+    for i in range(3):
+        rp, rv = ref.forward(x[i])
+        assert rel_l2(pol[i], rp) <= 2e-2 and rel_l2(val[i], rv) <= 2e-2
     pipe.close()
 
 

@@ -14,7 +14,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REF = "/root/reference"
 PATCH = os.path.join(ROOT, "integration", "leelaz-use-hip.patch")
-PATCHED = ["CMakeLists.txt", "src/config.h", "src/Network.cpp", "src/Network.h", "src/UCTSearch.cpp"]
+PATCHED = ["CMakeLists.txt", "src/Network.cpp", "src/Network.h", "src/UCTSearch.cpp"]
 
 need_ref = pytest.mark.skipif(not os.path.isdir(os.path.join(REF, "src")) or shutil.which("g++") is None,
                               reason="needs the reference tree and g++")
@@ -48,14 +48,18 @@ def test_patch_applies_and_the_patched_header_compiles_in_hip_mode(tmp_path):
     assert "std::make_unique<lzhip::HIPScheduler>" in net and '#include "forward_pipe.h"' in net
     cm = (tmp_path / "CMakeLists.txt").read_text()
     assert "option(USE_HIP" in cm and "target_link_libraries(leelaz lzhip)" in cm
-    # the patched Network.h with USE_HIP on (USE_OPENCL and USE_HALF stay defined, no OpenCL
-    # header is pulled in) together with the library's header
+    # the engine's run-time self-check against CPUPipe stays compiled in (config.h is not
+    # touched), and the search prints the library's batch counters where it printed OpenCL's
+    uct = (tmp_path / "src" / "UCTSearch.cpp").read_text()
+    assert "lzhip::batch_stats.single_evals" in uct and '#include "forward_pipe.h"' in uct
+    # the patched Network.h with USE_HIP on (USE_OPENCL, USE_HALF and the self-check stay
+    # defined, no OpenCL header is pulled in) together with the library's header
     tu = tmp_path / "hip_mode.cpp"
     tu.write_text('#include "config.h"\n#include "Network.h"\n#include "forward_pipe.h"\n'
-                  "#if !defined(USE_OPENCL) || !defined(USE_HALF) || defined(USE_OPENCL_SELFCHECK)\n"
+                  "#if !defined(USE_OPENCL) || !defined(USE_HALF) || !defined(USE_OPENCL_SELFCHECK)\n"
                   '#error "unexpected switches in a USE_HIP build"\n#endif\n'
                   "int main() { lzhip::HIPScheduler s(LZHIP_FP16, 8, 0); ForwardPipe* p = &s; "
-                  "return p == nullptr; }\n")
+                  "return p == nullptr || lzhip::batch_stats.batch_evals.load() != 0; }\n")
     r = syntax_only(["-DUSE_HIP", "-DLZHIP_ENGINE_BUILD", "-I", str(tmp_path / "src"),
                      "-I", os.path.join(REF, "src"), "-I", os.path.join(ROOT, "include")], str(tu))
     assert r.returncode == 0, r.stderr

@@ -18,11 +18,16 @@ def _pipe(pkg, netgen, blocks, filters, seed, precision, max_batch):
 
 
 @pytest.mark.parametrize("precision_name", ["FP32", "FP16"])
-def test_no_alloc_forward_matches_the_allocating_one(pkg, netgen, precision_name):
+@pytest.mark.parametrize("filters,max_batch", [(192, 8), (256, 8), (128, 64), (256, 64)])
+def test_no_alloc_forward_matches_the_allocating_one(pkg, netgen, precision_name, filters,
+                                                     max_batch):
+    """256 filters at max_batch 8 fill the static array exactly; a handle made for 64
+    positions has lane buffers with more tile rows per position than the static array
+    (the serving case: a large handle, small no-alloc calls)."""
     import torch
     precision = getattr(pkg, precision_name)
-    print("case: no-alloc forward", precision_name, flush=True)
-    pipe = _pipe(pkg, netgen, 3, 192, 91, precision, 8)
+    print("case: no-alloc forward", precision_name, filters, max_batch, flush=True)
+    pipe = _pipe(pkg, netgen, 3, filters, 91, precision, max_batch)
     x = netgen.synthetic_inputs(8, seed=92)
     d_in = torch.from_numpy(x).cuda()
     for n in (8, 3):    # the second call is smaller: the array still holds the first one's tiles
@@ -40,6 +45,43 @@ def test_no_alloc_forward_matches_the_allocating_one(pkg, netgen, precision_name
         assert np.array_equal(got_pol.cpu().numpy(), want_pol.cpu().numpy())
         assert np.array_equal(got_val.cpu().numpy(), want_val.cpu().numpy())
     pipe.close()
+
+
+def test_no_alloc_forwards_of_two_handles_share_the_array_in_turn(pkg, netgen):
+    """Two handles of different width and storage type on one GPU, their no-alloc forwards
+    enqueued alternately on their own streams with no host synchronisation in between: the
+    library orders them on the device, and each gives what its allocating forward gives."""
+    import torch
+    print("case: no-alloc, two handles", flush=True)
+    a = _pipe(pkg, netgen, 3, 256, 95, pkg.FP16, 8)
+    b = _pipe(pkg, netgen, 2, 64, 96, pkg.FP32, 8)
+    xa = torch.from_numpy(netgen.synthetic_inputs(8, seed=97)).cuda()
+    xb = torch.from_numpy(netgen.synthetic_inputs(5, seed=98)).cuda()
+    want = []
+    for pipe, x, n in ((a, xa, 8), (b, xb, 5)):
+        pol = torch.zeros(n, 722, device="cuda")
+        val = torch.zeros(n, 361, device="cuda")
+        torch.cuda.synchronize()
+        pipe.forward_batch_device(n, x.data_ptr(), pol.data_ptr(), val.data_ptr())
+        pipe.sync()
+        want.append((pol.cpu().numpy(), val.cpu().numpy()))
+    outs = [[(torch.full((8, 722), -7.0, device="cuda"), torch.full((8, 361), -7.0, device="cuda"))
+             for _ in range(6)] for _ in range(2)]
+    torch.cuda.synchronize()
+    for rep in range(6):
+        a.forward_batch_device_noalloc(8, xa.data_ptr(), outs[0][rep][0].data_ptr(),
+                                       outs[0][rep][1].data_ptr())
+        b.forward_batch_device_noalloc(5, xb.data_ptr(), outs[1][rep][0].data_ptr(),
+                                       outs[1][rep][1].data_ptr())
+    a.sync()
+    b.sync()
+    for rep in range(6):
+        assert np.array_equal(outs[0][rep][0].cpu().numpy(), want[0][0]), rep
+        assert np.array_equal(outs[0][rep][1].cpu().numpy(), want[0][1]), rep
+        assert np.array_equal(outs[1][rep][0].cpu().numpy()[:5], want[1][0]), rep
+        assert np.array_equal(outs[1][rep][1].cpu().numpy()[:5], want[1][1]), rep
+    a.close()
+    b.close()
 
 
 def test_no_alloc_forward_refuses_what_does_not_fit(pkg, netgen):
