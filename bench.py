@@ -280,7 +280,7 @@ def measure_forward(pkg, netgen, torch, blocks, F, precision, B, steps, warmup, 
     if host_buffers:
         # the same batch handed over as host buffers (pageable numpy arrays in and out): copy
         # to pinned staging, H2D, forward, D2H, copy out -- PCIe inside the timed region
-        host_steps = max(3, steps // 2)
+        host_steps = max(steps, min_block)       # at least 200 forwards unless --headline-only
         pipe.forward_batch(x)
         t0 = time.perf_counter()
         for _ in range(host_steps):
@@ -309,6 +309,22 @@ def measure_forward(pkg, netgen, torch, blocks, F, precision, B, steps, warmup, 
             "callers_as_lanes": (None if host2_dt is None else
                                  {"value": B / host2_dt, "callers": lanes,
                                   "note": "one calling thread per lane, a batch each at a time"})}
+
+        # Events on the stream around H2D (pinned) + tower + heads on the device + D2H
+        # (pinned), forwards one after the other on one lane: five blocks of at least 200
+        # forwards after 20 warm-up forwards, median.
+        pipe.push_heads(h)
+        per_block = max(steps, min_block)
+        pipe.timed_evaluations(x, 20)
+        ms_blocks = sorted(pipe.timed_evaluations(x, per_block)[0] for _ in range(5))
+        med = ms_blocks[2]
+        res["events_h2d_tower_heads_d2h"] = {
+            "value": B * per_block / (med * 1e-3), "unit": "evals/s",
+            "ms_per_forward": med / per_block, "forwards_per_block": per_block, "blocks": 5,
+            "min": B * per_block / (ms_blocks[-1] * 1e-3), "max": B * per_block / (ms_blocks[0] * 1e-3),
+            "note": "stream events around (copy of the planes from pinned host memory + tower + "
+                    "fully connected heads, softmax and tanh on the device + copy of policy and "
+                    "value to pinned host memory), one lane, median of five blocks"}
 
     # per-kernel-class device time, measured live with HIP events on the pipe's stream
     ms = np.zeros(pkg.K_COUNT)
@@ -399,28 +415,44 @@ def measure_forward(pkg, netgen, torch, blocks, F, precision, B, steps, warmup, 
 
 def copy_floor(torch, B, F, e):
     """What a plain device copy of the GEMM's tile arrays takes on this box: V-sized read +
-    M-sized write (36 x 25B x F elements each) per launch, launches back to back over three
-    buffer pairs, timed with events on the stream they run on."""
+    M-sized write (36 x 25B x F elements each) per launch, launches back to back, timed with
+    events on the stream they run on -- at three working sets: two arrays that swap roles
+    (resident in the 256 MB memory-side cache), three pairs (the working set of two lanes),
+    and enough pairs to pass 1 GB (every byte from and to HBM)."""
     n = 36 * 25 * B * F
     dt = torch.float16 if e == 2 else torch.float32
-    src = [torch.ones(n, dtype=dt, device="cuda") for _ in range(3)]
-    dst = [torch.empty(n, dtype=dt, device="cuda") for _ in range(3)]
-    for i in range(6):
-        dst[i % 3].copy_(src[i % 3])
-    torch.cuda.synchronize()
-    reps = 60
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(reps):
-        dst[(i + 1) % 3].copy_(src[i % 3])
-    e1.record()
-    torch.cuda.synchronize()
-    us = e0.elapsed_time(e1) * 1e3 / reps
     nbytes = 2.0 * n * e
-    return {"us_per_launch": us, "bytes_per_launch": nbytes, "achieved": nbytes / (us * 1e-6) / 1e9,
-            "unit": "GB/s", "frac_of_hbm_peak": nbytes / (us * 1e-6) / PEAK_HBM,
-            "note": "device-to-device copy of a V-sized array into an M-sized one (the bytes a "
-                    "GEMM launch moves, less the filters), launch to launch"}
+    out = {"bytes_per_launch": nbytes, "unit": "GB/s",
+           "note": "device-to-device copy of a V-sized array into an M-sized one (the bytes a "
+                   "GEMM launch moves, less the filters), launch to launch"}
+
+    def run(pairs, swap):
+        src = [torch.ones(n, dtype=dt, device="cuda") for _ in range(pairs)]
+        dst = src[::-1] if swap else [torch.empty(n, dtype=dt, device="cuda") for _ in range(pairs)]
+        k = len(src)
+        for i in range(2 * k):
+            dst[(i + 1) % k].copy_(src[i % k])
+        torch.cuda.synchronize()
+        reps = 60
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            dst[(i + 1) % k].copy_(src[i % k])
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        ws = (k if swap else 2 * k) * n * e
+        return {"working_set_mb": ws / 1e6, "us_per_launch": us,
+                "achieved": nbytes / (us * 1e-6) / 1e9,
+                "frac_of_hbm_peak": nbytes / (us * 1e-6) / PEAK_HBM}
+
+    big_pairs = int(0.55e9 // (n * e)) + 1
+    out["cache_resident"] = run(2, True)
+    out["two_lanes"] = run(3, False)
+    out["hbm_only"] = run(big_pairs, False)
+    # the figures earlier versions of this line carried, for the middle working set
+    out.update({k: out["two_lanes"][k] for k in ("us_per_launch", "achieved", "frac_of_hbm_peak")})
+    return out
 
 
 def side_config(pkg, netgen, torch, blocks, F, precision, B, args, cpu=False):
@@ -584,9 +616,20 @@ def main():
         "roofline_transforms": head["roofline_transforms"],
         "kernel_ms_per_forward": head["kernel_ms_per_forward"],
         "gemm_mfma_util_pct": 100.0 * head["roofline"]["frac"],
+        "events_h2d_tower_heads_d2h": head["events_h2d_tower_heads_d2h"],
         "hbm_copy_floor": copy_floor(torch, B, F, 2 if args.precision == "fp16" else 4),
         "cpu_baseline": cpu,
     }
+    # what this GEMM launch is against the copy rates measured above: the roof that applies
+    # to one lane is the cache-resident one (V, M and the activations of a lane are ~100 MB)
+    floor = out["hbm_copy_floor"]
+    alg = out["roofline"]["algorithmic_bytes_per_launch"]
+    us = out["roofline"]["avg_launch_us"]
+    out["roofline"]["hbm_view"]["vs_copy_rate"] = {
+        k: alg / (us * 1e-6) / 1e9 / floor[k]["achieved"]
+        for k in ("cache_resident", "two_lanes", "hbm_only")}
+    out["config"]["one_lane_evals_per_s"] = head["one_lane"]["value"]
+    out["config"]["events_h2d_tower_heads_d2h_evals_per_s"] = head["events_h2d_tower_heads_d2h"]["value"]
     if not args.headline_only:
         # the same network in fp32, and the three smaller configurations, one line each
         if args.precision == "fp16":

@@ -191,6 +191,16 @@ int lzhip_push_heads(lzhip_handle* h, const float* bn_pol_mean, const float* bn_
 int lzhip_evaluate_batch(lzhip_handle* h, int n, const float* in, float temperature,
                          float* policy, float* value, float* logits, float* pol, float* val);
 
+/* Measurement: `reps` evaluations of the same n positions one after the other on lane 0,
+ * each of them host-to-device copy of the planes (from pinned memory), tower, heads on
+ * the device, device-to-host copy of policy [n][362] and value [n] (to pinned memory),
+ * bracketed by two events on that stream; *ms = time between the events.  policy and
+ * value receive the last evaluation's results.  The counterpart of timing
+ * OpenCL_Network::forward from its first enqueueWriteBuffer to the end of its blocking
+ * read (reference src/OpenCL.cpp:208-216,312-318), heads included.  Needs lzhip_push_heads. */
+int lzhip_timed_evaluations(lzhip_handle* h, int n, int reps, const float* in,
+                            float temperature, float* policy, float* value, float* ms);
+
 /* One position through the batching queue with the heads computed on the
  * device: the whole of Network::get_output_internal's arithmetic (reference
  * src/Network.cpp:824-851) except the symmetry un-rotation, as one blocking,

@@ -39,7 +39,7 @@ EXPORTS = [
     "lzhip_forward_batch_device_lane", "lzhip_forward_batch_device_noalloc", "lzhip_sync", "lzhip_stream",
     "lzhip_drain", "lzhip_resume", "lzhip_get_stats", "lzhip_reset_stats",
     "lzhip_process_batch_stats", "lzhip_push_heads",
-    "lzhip_evaluate_batch", "lzhip_forward_eval", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
+    "lzhip_evaluate_batch", "lzhip_timed_evaluations", "lzhip_forward_eval", "lzhip_winograd_transform_f", "lzhip_process_bn_var",
     "lzhip_ceil_multiple",
     "lzhip_debug_layer", "lzhip_get_act_scales", "lzhip_profile_forward", "lzhip_last_error",
     "lzhip_version",
@@ -168,6 +168,8 @@ def lib():
         L.lzhip_push_heads.argtypes = [ctypes.c_void_p] + [_fp] * 10
         L.lzhip_evaluate_batch.argtypes = [ctypes.c_void_p, ctypes.c_int, _fp, ctypes.c_float] + [_fp] * 5
         L.lzhip_forward_eval.argtypes = [ctypes.c_void_p, _fp, ctypes.c_float, _fp, _fp]
+        L.lzhip_timed_evaluations.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, _fp,
+                                              ctypes.c_float, _fp, _fp, _fp]
         L.lzhip_winograd_transform_f.argtypes = [_fp, ctypes.c_int, ctypes.c_int, _fp]
         L.lzhip_process_bn_var.argtypes = [_fp, ctypes.c_int]
         L.lzhip_ceil_multiple.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
@@ -496,6 +498,19 @@ class HIPScheduler:
         if want_raw:
             return policy, value, logits, pol, val
         return policy, value, logits
+
+    def timed_evaluations(self, inputs, reps, temperature=1.0):
+        """`reps` evaluations (H2D + tower + device heads + D2H) of the same batch on one
+        lane between two stream events: returns (milliseconds, policy, value)."""
+        self._need()
+        x = _f32(inputs).reshape(-1, INPUT_SIZE)
+        n = x.shape[0]
+        policy = np.empty((n, MOVES), dtype=np.float32)
+        value = np.empty(n, dtype=np.float32)
+        ms = np.zeros(1, dtype=np.float32)
+        _check(lib().lzhip_timed_evaluations(self._h, n, int(reps), _ptr(x), float(temperature),
+                                             _ptr(policy), _ptr(value), _ptr(ms)))
+        return float(ms[0]), policy, value
 
     # -- callers above forward() ------------------------------------------------
     def get_output(self, heads, boards, to_move, symmetry=0, temperature=1.0):

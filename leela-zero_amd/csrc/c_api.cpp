@@ -271,6 +271,15 @@ int lzhip_evaluate_batch(lzhip_handle* h, int n, const float* in, float temperat
     GUARD_END
 }
 
+int lzhip_timed_evaluations(lzhip_handle* h, int n, int reps, const float* in,
+                            float temperature, float* policy, float* value, float* ms) {
+    if (!h || !in || !policy || !value || !ms) return fail(LZHIP_EINVAL, "null argument");
+    GUARD_BEGIN
+    *ms = h->pipe->timed_evaluations(n, reps, in, temperature, policy, value);
+    return LZHIP_OK;
+    GUARD_END
+}
+
 int lzhip_forward_eval(lzhip_handle* h, const float* in, float temperature, float* policy,
                        float* value) {
     if (!h || !in || !policy || !value) return fail(LZHIP_EINVAL, "null argument");

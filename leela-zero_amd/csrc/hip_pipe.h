@@ -49,6 +49,13 @@ public:
     virtual void evaluate_batch(int n, const float* in, float temperature, float* policy,
                                 float* value, float* logits, float* pol, float* val) = 0;
 
+    // `reps` evaluations of one batch, one after the other on lane 0, each of them the
+    // copy of the planes from pinned host memory, the tower, the heads and the copy of
+    // policy and value back to pinned host memory; returns the milliseconds between two
+    // events recorded on that stream around all of them.
+    virtual float timed_evaluations(int n, int reps, const float* in, float temperature,
+                                    float* policy, float* value) = 0;
+
     virtual void debug_layer(int layer, int n, const float* act_in, const float* res, float* V,
                              float* M, float* Y) = 0;
     virtual void profile_forward(int n, const float* d_in, float* d_pol, float* d_val,

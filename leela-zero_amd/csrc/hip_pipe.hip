@@ -531,6 +531,46 @@ public:
             HIP_CHECK(hipMemcpy(val, m_dval.p, sizeof(float) * (size_t)n * kPts, hipMemcpyDeviceToHost));
     }
 
+    float timed_evaluations(int n, int reps, const float* in, float temperature, float* policy,
+                            float* value) override {
+        Lane& ln = m_lane[0];
+        std::lock_guard<std::mutex> lk(ln.mu);
+        check_ready(n);
+        if (!m_heads_ready) throw std::invalid_argument("push_heads has not been called");
+        if (!(temperature > 0.0f)) throw std::invalid_argument("temperature must be positive");
+        if (reps < 1 || reps > 100000) throw std::invalid_argument("reps out of range");
+        HIP_CHECK(hipSetDevice(m_device));
+        const size_t in_count = (size_t)n * kInPlanes * kPts;
+        PinnedBuf<float> hin, hpolicy, hvalue;
+        hin.alloc(in_count);
+        hpolicy.alloc((size_t)n * 362);
+        hvalue.alloc((size_t)n);
+        std::memcpy(hin.p, in, in_count * sizeof(float));
+        HeadParams hp{m_h[0].p, m_h[1].p, m_h[2].p, m_h[3].p, m_h[4].p,
+                      m_h[5].p, m_h[6].p, m_h[7].p, m_h[8].p, m_h[9].p};
+        HIP_CHECK(hipStreamSynchronize(ln.stream));
+        HIP_CHECK(hipEventRecord(m_ev_start[0], ln.stream));
+        for (int r = 0; r < reps; r++) {
+            HIP_CHECK(hipMemcpyAsync(m_din.p, hin.p, in_count * sizeof(float),
+                                     hipMemcpyHostToDevice, ln.stream));
+            run_forward(ln, n, m_din.p, nullptr, m_dpol.p, m_dval.p);
+            launch_heads(m_dpol.p, m_dval.p, hp, temperature, m_dpolicy.p, nullptr, m_dvalue.p,
+                         m_dwork.p, n, ln.stream);
+            HIP_CHECK(hipMemcpyAsync(hpolicy.p, m_dpolicy.p, sizeof(float) * (size_t)n * 362,
+                                     hipMemcpyDeviceToHost, ln.stream));
+            HIP_CHECK(hipMemcpyAsync(hvalue.p, m_dvalue.p, sizeof(float) * (size_t)n,
+                                     hipMemcpyDeviceToHost, ln.stream));
+        }
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipEventRecord(m_ev_stop[0], ln.stream));
+        HIP_CHECK(hipEventSynchronize(m_ev_stop[0]));
+        float ms = 0.0f;
+        HIP_CHECK(hipEventElapsedTime(&ms, m_ev_start[0], m_ev_stop[0]));
+        std::memcpy(policy, hpolicy.p, sizeof(float) * (size_t)n * 362);
+        std::memcpy(value, hvalue.p, sizeof(float) * (size_t)n);
+        return ms;
+    }
+
     // -------------------------------------------------------------------
     void debug_layer(int layer, int n, const float* act_in, const float* res, float* Vout,
                      float* Mout, float* Yout) override {
