@@ -430,14 +430,15 @@ def copy_floor(torch, B, F, e):
         src = [torch.ones(n, dtype=dt, device="cuda") for _ in range(pairs)]
         dst = src[::-1] if swap else [torch.empty(n, dtype=dt, device="cuda") for _ in range(pairs)]
         k = len(src)
+        into = (lambda i: dst[i % k]) if swap else (lambda i: dst[(i + 1) % k])
         for i in range(2 * k):
-            dst[(i + 1) % k].copy_(src[i % k])
+            into(i).copy_(src[i % k])
         torch.cuda.synchronize()
         reps = 60
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for i in range(reps):
-            dst[(i + 1) % k].copy_(src[i % k])
+            into(i).copy_(src[i % k])
         e1.record()
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / reps
