@@ -161,7 +161,10 @@ public:
             bool armed = true;
             ~Unwind() { if (armed) self->release_device_objects(); }
         } unwind{this};
-        for (int i = 0; i < m_n_lanes; i++) HIP_CHECK(hipStreamCreate(&m_lane[i].stream));
+        for (int i = 0; i < m_n_lanes; i++) {
+            HIP_CHECK(hipStreamCreate(&m_lane[i].stream));
+            HIP_CHECK(hipEventCreateWithFlags(&m_lane[i].last, hipEventDisableTiming));
+        }
         const size_t B = (size_t)max_batch;
         m_din.alloc(B * kInPlanes * kPts);
         m_dpol.alloc(B * 2 * kPts);
@@ -183,7 +186,12 @@ public:
             for (auto& a : ln.act) a.alloc(B * kPts * m_Fp);
             ln.V.alloc((size_t)kPos * m_Tp * m_Fp);
             ln.M.alloc((size_t)kPos * m_Tp * m_Fp);
+            ln.flags.alloc(B * kFusedFlagsPerBoard);    // zeroed: no launch has epoch 0
         }
+        m_gave_up.alloc(1);
+        *m_gave_up.p = 0;
+        // measurement knob: 0 never, 1 when the forward is alone on the device, 2 always
+        if (const char* e = std::getenv("LZHIP_FUSE")) m_fuse = std::atoi(e);
         m_scalar.alloc(4);
         for (int i = 0; i < kTimerPool; i++) {
             HIP_CHECK(hipEventCreate(&m_ev_start[i]));
@@ -211,6 +219,8 @@ public:
             sl.done = nullptr;
         }
         for (auto& ln : m_lane) {
+            if (ln.last) (void)hipEventDestroy(ln.last);
+            ln.last = nullptr;
             if (ln.stream) (void)hipStreamDestroy(ln.stream);
             ln.stream = nullptr;
         }
@@ -373,6 +383,16 @@ public:
     void sync() override {
         HIP_CHECK(hipSetDevice(m_device));
         for (int i = 0; i < m_n_lanes; i++) HIP_CHECK(hipStreamSynchronize(m_lane[i].stream));
+        check_waits();
+    }
+
+    // A fused launch whose work-groups gave up waiting for each other has produced nothing
+    // usable; it says so through a word in mapped host memory.
+    void check_waits() {
+        if (__atomic_load_n(m_gave_up.p, __ATOMIC_RELAXED) != 0)
+            throw std::runtime_error(
+                "a fused transform + GEMM launch ran into its wait limit: the results of this "
+                "handle are invalid (LZHIP_FUSE=0 runs the two kernels as separate launches)");
     }
 
     // Host-buffer forward.  Up to kIoSlots callers may be inside at once: each
@@ -466,6 +486,7 @@ public:
             HIP_CHECK(hipEventRecord(sl->done, ln.stream));
         }
         HIP_CHECK(hipEventSynchronize(sl->done));
+        check_waits();
         std::memcpy(out_a, sl->hpol.p, sizeof(float) * (size_t)n * na);
         std::memcpy(out_b, sl->hval.p, sizeof(float) * (size_t)n * nb);
     }
@@ -668,6 +689,9 @@ private:
         hipStream_t stream = nullptr;
         std::mutex mu;  // serialises enqueues on this lane
         DevBuf<P> act0, act[3], V, M;
+        DevBuf<unsigned long long> flags;   // fused launches: one word per (board, channel group)
+        unsigned long long epoch = 0;       // grows by one per fused launch (under mu)
+        hipEvent_t last = nullptr;          // recorded behind the lane's latest forward
         std::map<GraphKey, hipGraphExec_t> graphs;
     };
     static constexpr int kLanes = 3;   // upper bound; m_n_lanes are in use
@@ -678,6 +702,10 @@ private:
         hipStream_t stream = nullptr;
         P *act0 = nullptr, *act[3] = {nullptr, nullptr, nullptr}, *V = nullptr, *M = nullptr;
         int Tp = 0;
+        // what a fused transform + GEMM launch synchronises through; null: separate launches
+        unsigned long long* flags = nullptr;
+        unsigned long long* epoch = nullptr;
+        bool alone = false;   // no other lane had work on the device when this one was enqueued
     };
     Work work_of(Lane& ln) const {
         Work w;
@@ -687,6 +715,13 @@ private:
         w.V = ln.V.p;
         w.M = ln.M.p;
         w.Tp = m_Tp;
+        w.flags = ln.flags.p;
+        w.epoch = &ln.epoch;
+        // (an event that was never recorded reads as complete)
+        w.alone = true;
+        for (int i = 0; i < m_n_lanes; i++)
+            if (&m_lane[i] != &ln && hipEventQuery(m_lane[i].last) != hipSuccess) w.alone = false;
+        (void)hipGetLastError();   // hipErrorNotReady is an answer, not a failure
         return w;
     }
 
@@ -784,6 +819,9 @@ private:
     void enqueue_forward(Lane& ln, int n, const float* d_in, const uint32_t* d_bits,
                          float* d_pol, float* d_val, bool timed) {
         enqueue_forward(work_of(ln), n, d_in, d_bits, d_pol, d_val, timed);
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        HIP_CHECK(hipStreamIsCapturing(ln.stream, &cap));
+        if (cap == hipStreamCaptureStatusNone) HIP_CHECK(hipEventRecord(ln.last, ln.stream));
     }
     void enqueue_forward(const Work& w, int n, const float* d_in, const uint32_t* d_bits,
                          float* d_pol, float* d_val, bool timed) {
@@ -796,11 +834,23 @@ private:
             launch_pack_input_bits<P>(d_bits, w.act0, n, kInPlanes, m_C0p, w.stream,
                                       timer(timed, LZHIP_K_PACK));
         launch_in_transform<P>(w.act0, w.V, n, m_C0p, w.Tp, w.stream, timer(timed, LZHIP_K_IN));
+        // Up to 32 boards (fp16, 256 filters) the transform of layer l and the GEMM of layer
+        // l + 1 go out as one launch when this forward has the device to itself: the fused
+        // launch shortens a chain of dependent kernels (one lane: +18 % evaluations/s at one
+        // board, +4..8 % at 4 to 32), but its waiting work-groups hold compute units that
+        // another lane's kernels would otherwise use (three lanes at 8 boards: -20 %).  Both
+        // ways give the same bits.  Not under graph capture (the launch carries a number that
+        // has to differ from launch to launch), not when every launch is timed, and not on
+        // the static working memory.
+        bool fused = false;
+        if constexpr (sizeof(P) == 2)
+            fused = m_fuse > 0 && (w.alone || m_fuse > 1) && !timed && !m_use_graph &&
+                    w.flags != nullptr && xform_gemm_shape(n, m_Fp, 2);
         int cur = 0, nxt = 1;  // block input (skip) / block output
+        launch_gemm<P>(w.V, m_layers[0].U.p, m_layers[0].Uf.p, w.M, Tu, w.Tp, m_layers[0].Cp, m_Fp,
+                       w.stream, timer(timed, LZHIP_K_GEMM));
         for (int l = 0; l < nl; l++) {
             Layer& L = m_layers[l];
-            launch_gemm<P>(w.V, L.U.p, L.Uf.p, w.M, Tu, w.Tp, L.Cp, m_Fp, w.stream,
-                           timer(timed, LZHIP_K_GEMM));
             const bool block_end = (l % 2) == 0;      // layer 0 and second convs
             const P* res = (block_end && l >= 2) ? w.act[cur] : nullptr;
             P* out = l == 0 ? w.act[cur] : w.act[nxt];
@@ -810,9 +860,23 @@ private:
                 launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, w.stream,
                                     timer(timed, LZHIP_K_HEAD));
             } else {
-                launch_out_in_transform<P>(w.M, res, block_end ? out : nullptr, w.V, L.d_scale.p,
-                                           L.d_mean.p, L.rfac, n, m_Fp, w.Tp, w.stream,
-                                           timer(timed, LZHIP_K_OUTIN));
+                Layer& N = m_layers[l + 1];
+                bool done = false;
+                if constexpr (sizeof(P) == 2) {
+                    if (fused) {
+                        launch_xform_gemm(w.M, res, block_end ? out : nullptr, w.V, L.d_scale.p,
+                                          L.d_mean.p, L.rfac, n, m_Fp, w.Tp, N.Uf.p, w.flags,
+                                          ++*w.epoch, m_gave_up.p, w.stream);
+                        done = true;
+                    }
+                }
+                if (!done) {
+                    launch_out_in_transform<P>(w.M, res, block_end ? out : nullptr, w.V,
+                                               L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, w.Tp,
+                                               w.stream, timer(timed, LZHIP_K_OUTIN));
+                    launch_gemm<P>(w.V, N.U.p, N.Uf.p, w.M, Tu, w.Tp, N.Cp, m_Fp, w.stream,
+                                   timer(timed, LZHIP_K_GEMM));
+                }
             }
             if (block_end && l >= 2) { const int o = cur; cur = nxt; nxt = o; }
         }
@@ -930,6 +994,8 @@ private:
     int m_timer_used = 0;
     LaunchTimer m_timer;
     bool m_use_graph = std::getenv("LZHIP_GRAPH") != nullptr;
+    int m_fuse = 1;                      // fused transform + GEMM launches (see enqueue_forward)
+    PinnedBuf<unsigned> m_gave_up;       // set by a fused launch whose wait ran into its limit
 };
 
 std::unique_ptr<HIPPipe> create_hip_pipe(int device, int precision, int max_batch, int filters) {

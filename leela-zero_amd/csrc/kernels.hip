@@ -20,6 +20,11 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 
 #define SQ2 1.4142135623730951f
+// Timeline hook for measurement builds (a harness that includes this file defines it to
+// record a timestamp); expands to nothing in the library.
+#ifndef LZ_STAMP
+#define LZ_STAMP(i)
+#endif
 constexpr int kStoreThrough = 17;  // cache policy of a raw buffer store: sc0 | sc1 (write-through)
 
 // ---------------------------------------------------------------------------
@@ -455,16 +460,22 @@ template <int CG> constexpr int xform_store_policy() { return CG == 64 ? kStoreT
 constexpr int kPlane = 22;       // LDS plane: 19 points + 1 zero halo before + 2 after
 constexpr int fuse_waves(int cg) { return (kTilesPerBoard + 128 / cg - 1) / (128 / cg); }
 
-template <typename P, int CG>
-__global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
-    const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ act_out,
-    P* __restrict__ Vn, const float* __restrict__ bn_scale, const float* __restrict__ bn_mean,
-    float rfac, int n, int Kp, int Tp) {
+// The body of the kernel, for work-group `wg` of the launch's transform work-groups, with
+// the LDS plane handed in (kPlane * kPlane * CG / 2 channel pairs); returns the work item
+// (board * channel groups + channel group) it processed, or -1 if `wg` had none.
+// VPOL = cache policy of the stores of V.  VSLAB: V is written channel group by channel
+// group, [36][Kp / CG][Tp][CG], instead of [36][Tp][Kp]: the 25 tiles of this work-group's
+// board and channel group are then one contiguous run per Winograd position (whole lines,
+// which is what makes write-through stores cheap), for a consumer that knows (xform_gemm_k).
+template <typename P, int CG, int VPOL, bool VSLAB = false>
+__device__ __forceinline__ int out_in_transform_body(
+    typename BufIO2<P>::pair_t* ybuf, unsigned wg, const P* M, const P* res, P* act_out, P* Vn,
+    const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int n,
+    int Kp, int Tp) {
     typedef typename BufIO2<P>::pair_t pair_t;
     constexpr int CP = CG / 2;        // channel pairs per plane cell = lanes per tile
     constexpr int TPW = 64 / CP;      // tiles per wavefront
     constexpr int WAVES = fuse_waves(CG);
-    __shared__ pair_t ybuf[kPlane * kPlane * CP];
     // Work-group w runs on die w % 8, each die with its own L2.  The narrow shapes share
     // 128-byte lines between the work-groups of neighbouring channel groups, so the items
     // (board, channel group) are cut into 8 contiguous segments and work-group w takes item
@@ -472,8 +483,8 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     // once, instead of once for each die that holds a piece of it.
     const int ncg = Kp / CG;
     const int per_die = (n * ncg + 7) >> 3;
-    const int item = (int)(blockIdx.x & 7) * per_die + (int)(blockIdx.x >> 3);
-    if (item >= n * ncg) return;
+    const int item = (int)(wg & 7) * per_die + (int)(wg >> 3);
+    if (item >= n * ncg) return -1;
     const int b = item / ncg;
     const int cg = item - b * ncg;
 
@@ -546,6 +557,7 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    LZ_STAMP(1);
     // zero the halo cells of the plane (rows and columns 0, 20, 21): 3 full rows
     // and 3 cells in each of the 19 rows between them; one cell per tile slot
     {
@@ -607,7 +619,9 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
             }
         }
     }
+    LZ_STAMP(2);
     __syncthreads();
+    LZ_STAMP(3);
     // The activation leaves only now: stores issued before the barrier would have to be
     // acknowledged before any wavefront may pass it; here they drain under phase 2.
     if (act_out != nullptr) {
@@ -648,15 +662,33 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
                 else outp[q].y = (P)d[q];
             }
         }
+        LZ_STAMP(4);
         if (valid) {
-            unsigned so = soff_t;
+            unsigned so = soff_t, vo = voff_t;
+            if constexpr (VSLAB) {
+                vo = cl * 2 * esz + sub * (unsigned)CG * esz;
+                so = ((unsigned)cg * (unsigned)Tp + (unsigned)(b * kTilesPerBoard + TPW * wave)) *
+                     (unsigned)CG * esz;
+            }
 #pragma unroll
             for (int p = 0; p < 36; p++) {
-                BufIO2<P>::template store<xform_store_policy<CG>()>(outp[p], rV, voff_t, so);
+                BufIO2<P>::template store<VPOL>(outp[p], rV, vo, so);
                 so += pstride;
             }
         }
     }
+    LZ_STAMP(5);
+    return item;
+}
+
+template <typename P, int CG>
+__global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
+    const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ act_out,
+    P* __restrict__ Vn, const float* __restrict__ bn_scale, const float* __restrict__ bn_mean,
+    float rfac, int n, int Kp, int Tp) {
+    __shared__ typename BufIO2<P>::pair_t ybuf[kPlane * kPlane * (CG / 2)];
+    (void)out_in_transform_body<P, CG, xform_store_policy<CG>()>(ybuf, blockIdx.x, M, res, act_out, Vn, bn_scale, bn_mean,
+                                       rfac, n, Kp, Tp);
 }
 
 template <typename P>
@@ -1437,12 +1469,32 @@ __host__ __device__ constexpr int gemm_stream_channel(int i) {
     return 16 * (i >> 4) + 8 * ((i >> 2) & 1) + 4 * ((i >> 3) & 1) + (i & 3);
 }
 
-template <int NKC, int NBLK, int NW>
-__global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __restrict__ V,
-                                                          const half_t* __restrict__ Uf,
-                                                          half_t* __restrict__ M, int T, int Tp,
-                                                          int Kp, int chunks, int nblk_total,
-                                                          int tiles_n, int seg) {
+// What a fused launch hands the GEMM's work-groups to wait on (see xform_gemm_k): one
+// 64-bit word per (board, channel group) of the transform that produces V in the same
+// launch, set to `epoch` when that work-group's stores have reached memory.
+struct StreamWait {
+    const unsigned long long* flags;
+    unsigned long long epoch;
+    unsigned* gave_up;     // set to 1 if a wait ran into its spin limit
+    int ncg;               // channel groups per board
+    int delay;             // pauses (of ~0.25 us) between the requests of a wavefront's filters
+};
+constexpr int kFlagSpinLimit = 1 << 18;   // polls of ~0.3 us each before a wait gives up
+
+// LDS of the streaming GEMM in halves: the ring of V blocks (as many stages as the
+// pipeline can use) and two copies of a block's result.
+template <int NKC, int NBLK, int NW> constexpr int gemm_stream_lds_halves() {
+    return (NBLK < 3 ? NBLK : 3) * 32 * (NKC * 16 + 8) + 2 * 32 * (32 * NW + 8);
+}
+
+// FUSED: the work-group is part of a fused launch (xform_gemm_k): it waits for the producers
+// of its rows, and reads V in the layout they write, [Kp / SLAB][Tp][SLAB] per position.
+template <int NKC, int NBLK, int NW, bool FUSED, int SLAB = 0>
+__device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg, const half_t* V,
+                                                      const half_t* __restrict__ Uf, half_t* M,
+                                                      int T, int Tp, int Kp, int chunks,
+                                                      int nblk_total, int tiles_n, int seg,
+                                                      StreamWait wait) {
     constexpr int D = kStreamAhead;
     constexpr int NT = 64 * NW;                  // threads: NW wavefronts of 32 output channels
     constexpr int CW = 32 * NW;                  // width of the column tile
@@ -1458,13 +1510,14 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
     constexpr int OSTAGE = 32 * OROW;
     static_assert(NKC % 2 == 0 && D == 2, "pipeline shape");
 
-    __shared__ __attribute__((aligned(16))) half_t smem[3 * STAGE + 2 * OSTAGE];
-    half_t* const obuf = smem + 3 * STAGE;
+    constexpr int NST = NBLK < 3 ? NBLK : 3;     // stages of the ring in use
+    static_assert(NST * STAGE + 2 * OSTAGE == gemm_stream_lds_halves<NKC, NBLK, NW>(), "LDS size");
+    half_t* const obuf = smem + NST * STAGE;
 
     const int n_items = kPos * chunks * tiles_n;
-    const int xcd = blockIdx.x & 7;
-    const int item = xcd * seg + (blockIdx.x >> 3);
-    if ((int)(blockIdx.x >> 3) >= seg || item >= n_items) return;
+    const int xcd = wg & 7;
+    const int item = xcd * seg + (int)(wg >> 3);
+    if ((int)(wg >> 3) >= seg || item >= n_items) return;
     const int tn = item % tiles_n;
     const int rest = item / tiles_n;
     const int ch = rest % chunks;
@@ -1481,25 +1534,48 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
     // chunk coordinates of this thread's loads within a block
     int lrow[CH], lcc[CH];
     bool lval[CH];
+    unsigned lslab[CH];   // slab layout: byte offset of the chunk's slab and place in its row
 #pragma unroll
     for (int i = 0; i < CH; i++) {
         const int idx = tid + i * NT;
         lval[i] = FULL || idx < NCH;
-        lrow[i] = (idx / CPRW) & 31;
-        lcc[i] = idx % CPRW;
+        if constexpr (SLAB > 0) {
+            // a wavefront's 64 chunks are consecutive rows of one slab: one contiguous KiB
+            constexpr int CPS = SLAB / 8;               // chunks per row of a slab
+            const int g = idx / (32 * CPS), rem = idx % (32 * CPS);
+            lrow[i] = rem / CPS;
+            lcc[i] = g * CPS + rem % CPS;
+            lslab[i] = ((unsigned)g * (unsigned)Tp * SLAB + (unsigned)(rem % CPS) * 8u) * 2u;
+        } else {
+            lrow[i] = (idx / CPRW) & 31;
+            lcc[i] = idx % CPRW;
+            lslab[i] = 0;
+        }
     }
     const half_t* Vp = V + (size_t)p * Tp * Cp;
 
     int4v st[D][CH];
+    // In a fused launch V has just been written by work-groups of the same launch on other
+    // dies: its loads carry the device-scope policy (sc1), which takes them past this
+    // die's caches to where those (written-through) stores went.
+    const __amdgpu_buffer_rsrc_t rV = make_rsrc(Vp, (size_t)Tp * Cp * sizeof(half_t));
     auto gload = [&](int slot, int s) {
         // steps past the last real block re-read that block (cache hits, never stored)
         const int blk = blk0 + (s < nreal ? s : nreal - 1);
 #pragma unroll
         for (int i = 0; i < CH; i++) {
             const int row = min(blk * 32 + lrow[i], T - 1);
-            if (lval[i])
-                st[slot][i] =
-                    *reinterpret_cast<const int4v*>(Vp + (size_t)row * Cp + lcc[i] * 8);
+            if (lval[i]) {
+                if constexpr (SLAB > 0)
+                    st[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rV, lslab[i] + (unsigned)row * (unsigned)(SLAB * 2), 0, 16);
+                else if constexpr (FUSED)
+                    st[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rV, (unsigned)(row * Cp + lcc[i] * 8) * 2u, 0, 16);
+                else
+                    st[slot][i] =
+                        *reinterpret_cast<const int4v*>(Vp + (size_t)row * Cp + lcc[i] * 8);
+            }
         }
     };
     auto lstore = [&](int slot, int buf) {
@@ -1514,12 +1590,48 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
     // wait for V only, and each matrix instruction of the first step only for the filter
     // fragments up to its own, so the first step starts while most of U is still arriving:
     // -0.5 us per launch at 64 boards against U first.)
-    gload(0, 0);
-    if (NBLK > 1) gload(1, 1);
     int4v u[NKC];
-    {
-        const half_t* Up =
-            Uf + ((((size_t)p * (Kp / 32) + (size_t)tn * NW + wave) * NKC) * 64 + lane) * 8;
+    const half_t* Up =
+        Uf + ((((size_t)p * (Kp / 32) + (size_t)tn * NW + wave) * NKC) * 64 + lane) * 8;
+    if constexpr (FUSED) {
+        // The filters depend on nothing in this launch: they are requested first and
+        // arrive while the transform work-groups are still producing V.  Then wait for the
+        // transform work-groups of every board that has a tile among this work-group's rows.
+#pragma unroll
+        for (int kc = 0; kc < NKC; kc++) {
+            u[kc] = *reinterpret_cast<const int4v*>(Up + (size_t)kc * 64 * 8);
+            if (wait.delay > 0) {
+                // one KiB per wavefront at a time: the transform work-group that shares this
+                // compute unit's memory pipeline is the one everything here waits for
+                __builtin_amdgcn_sched_barrier(0);
+                for (int q = 0; q < wait.delay; q++) __builtin_amdgcn_s_sleep(8);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        LZ_STAMP(10);
+        const int row_lo = blk0 * 32, row_hi = min(blk1 * 32, T);
+        const int b_lo = row_lo / kTilesPerBoard, b_hi = (row_hi - 1) / kTilesPerBoard;
+        const int nflags = (b_hi - b_lo + 1) * wait.ncg;
+        const unsigned long long* f = wait.flags + (size_t)b_lo * wait.ncg;
+        for (int i = tid; i < nflags; i += NT) {
+            int polls = 0;
+            while (__hip_atomic_load(f + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) !=
+                   wait.epoch) {
+                __builtin_amdgcn_s_sleep(2);
+                if (++polls > kFlagSpinLimit) {   // never hang: report and go on
+                    __hip_atomic_store(wait.gave_up, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_SYSTEM);
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+        LZ_STAMP(11);
+        gload(0, 0);
+        if (NBLK > 1) gload(1, 1);
+    } else {
+        gload(0, 0);
+        if (NBLK > 1) gload(1, 1);
 #pragma unroll
         for (int kc = 0; kc < NKC; kc++)
             u[kc] = *reinterpret_cast<const int4v*>(Up + (size_t)kc * 64 * 8);
@@ -1527,6 +1639,7 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
     lstore(0, 0);
     if (NBLK > 1) lstore(1, 1);
     __syncthreads();
+    LZ_STAMP(12);
 
     // M goes out through a raw buffer whose extent is the T real rows of this position:
     // rows past the last tile, and the steps past this work-group's last block, get an
@@ -1613,8 +1726,85 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
         *reinterpret_cast<half8v*>(O) = o0;
         *reinterpret_cast<half8v*>(O + 16) = o1;
         __syncthreads();
+        LZ_STAMP(13 + s);
     }
     send_rows(NBLK - 1);
+}
+
+template <int NKC, int NBLK, int NW>
+__global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __restrict__ V,
+                                                          const half_t* __restrict__ Uf,
+                                                          half_t* __restrict__ M, int T, int Tp,
+                                                          int Kp, int chunks, int nblk_total,
+                                                          int tiles_n, int seg) {
+    __shared__ __attribute__((aligned(16))) half_t smem[gemm_stream_lds_halves<NKC, NBLK, NW>()];
+    wino_gemm_stream_body<NKC, NBLK, NW, false>(smem, blockIdx.x, V, Uf, M, T, Tp, Kp, chunks,
+                                                nblk_total, tiles_n, seg, StreamWait{});
+}
+
+// ---------------------------------------------------------------------------
+// One launch for the fused transform of layer l (M_l -> V_{l+1}) and the GEMM of layer l+1
+// (V_{l+1} -> M_{l+1}), for small batches.  Two dependent launches cost a hand-over of
+// ~2.4 us between them whatever their size, and a GEMM work-group spends its first ~2 us
+// fetching 128 KiB of filters that depend on nothing: at 16 boards those two are a third of
+// a layer.  Here the launch's first work-groups run the transform and the rest the GEMM.
+// The GEMM work-groups request their filters at once, then wait, per board whose tiles
+// they multiply, for a word that each transform work-group sets (to the launch's `epoch`,
+// a number that grows with every fused launch of a lane, so nothing has to be cleared)
+// after its stores of V -- written through, with the device-scope policy -- have been
+// acknowledged; the GEMM work-groups read V with the same policy.  (Release and acquire
+// fences in their place would write back and invalidate a die's whole L2 once per wavefront:
+// measured 60 us per launch at 16 boards.)  With up to 16 boards both kinds of work-group
+// fit a compute unit together (4 + 8 wavefronts, 168 registers each, 2 x 67 KiB of LDS),
+// so the filters arrive under the transform; with more they follow as the transform's
+// work-groups retire, and the launch still saves the hand-over.
+//
+// Waiting is safe because the waiters never hold what the producers need: work-groups are
+// dispatched in the order of their index, so every transform work-group is resident (or
+// done) before the first GEMM work-group starts, and a transform work-group waits for
+// nothing.  A wait is bounded all the same: after kFlagSpinLimit polls it reports through
+// `gave_up` and goes on, so that the launch always ends.
+//
+// Inside such a launch V is laid out channel group by channel group ([36][Kp / CG][Tp][CG],
+// see out_in_transform_body): nothing outside the launch reads it.
+//
+// The buffers: the transform reads M and writes V, the GEMM reads V and writes M -- the
+// same M.  A GEMM work-group writes rows of M only after every transform work-group of
+// the boards those rows belong to has finished, i.e. after their last read.
+template <int CG, int NBLK, int NW>
+__global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) void xform_gemm_k(
+    half_t* M, const half_t* res, half_t* act_out, half_t* V, const float* __restrict__ bn_scale,
+    const float* __restrict__ bn_mean, float rfac, int n, int Kp, int Tp,
+    const half_t* __restrict__ Uf, int T, int chunks, int nblk_total, int tiles_n, int seg,
+    unsigned n_xform_wg, unsigned long long* flags, unsigned long long epoch, unsigned* gave_up,
+    int delay) {
+    typedef BufIO2<half_t>::pair_t pair_t;
+    constexpr int NKC = 2 * NW;      // tower layers: as many input as output channels
+    constexpr int XBYTES = kPlane * kPlane * (CG / 2) * (int)sizeof(pair_t);
+    constexpr int GBYTES = gemm_stream_lds_halves<NKC, NBLK, NW>() * 2;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[XBYTES > GBYTES ? XBYTES : GBYTES];
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    LZ_STAMP(0);
+    if (blockIdx.x < n_xform_wg) {
+        if (wave >= fuse_waves(CG)) return;    // the block is sized for the larger role
+        const int item = out_in_transform_body<half_t, CG, kStoreThrough, true>(
+            reinterpret_cast<pair_t*>(lds), blockIdx.x, M, res, act_out, V, bn_scale, bn_mean,
+            rfac, n, Kp, Tp);
+        if (item < 0) return;                  // uniform over the work-group
+        // V was stored write-through: once a wavefront's stores are acknowledged they are in
+        // memory, past every die's cache.  All wavefronts wait for that, then one word says so.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        LZ_STAMP(6);
+        __syncthreads();
+        if (threadIdx.x == 0)
+            __hip_atomic_store(flags + item, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        LZ_STAMP(7);
+    } else {
+        if (wave >= NW) return;
+        wino_gemm_stream_body<NKC, NBLK, NW, true, CG>(
+            reinterpret_cast<half_t*>(lds), blockIdx.x - n_xform_wg, V, Uf, M, T, Tp, Kp, chunks,
+            nblk_total, tiles_n, seg, StreamWait{flags, epoch, gave_up, Kp / CG, delay});
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1900,6 +2090,60 @@ static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int
         case 192: launch_gemm_stream_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
         default: launch_gemm_stream_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
     }
+}
+
+// Shapes served by the fused transform + GEMM launch: fp16 towers of 256 filters with the
+// narrow transform shapes (up to 32 boards).
+bool xform_gemm_shape(int n, int Kp, int elem_bytes) {
+    return elem_bytes == 2 && Kp == 256 && n >= 1 && n * (Kp / 64) <= 128;
+}
+
+// Pauses between a GEMM wavefront's 16 filter requests in a fused launch.  Requested all at
+// once, 128 KiB per compute unit go through the memory pipeline that the transform
+// work-group on the same unit is using, and that work-group is what the launch waits for
+// (measured at 16 boards: the slowest transform work-group ends at 10.2 us instead of
+// 8.9, the launch takes 18.1 us instead of 16.6).  Spread out, the filters still arrive
+// before V is ready: two pauses per request from 12 boards (the transform then takes
+// ~9 us), one from 6, none below (its 4 us leave no time to spread anything) and none above
+// 16 boards, where the GEMM work-groups only start when the transform's have left.
+static int fused_filter_pauses(int n) { return n > 16 ? 0 : n >= 12 ? 2 : n >= 6 ? 1 : 0; }
+
+template <int CG, int NBLK, int NW>
+static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, half_t* V,
+                                 const float* bn_scale, const float* bn_mean, float rfac, int n,
+                                 int Kp, int Tp, const half_t* Uf, unsigned long long* flags,
+                                 unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
+    const int T = n * kTilesPerBoard;
+    const int nblk = (T + 31) / 32;
+    const int chunks = (nblk + NBLK - 1) / NBLK;
+    const int tiles_n = Kp / (32 * NW);
+    const int seg = (kPos * chunks * tiles_n + 7) / 8;
+    const unsigned n_xform_wg = 8u * (unsigned)((n * (Kp / CG) + 7) / 8);
+    constexpr int WAVES = NW > fuse_waves(CG) ? NW : fuse_waves(CG);
+    hipLaunchKernelGGL((xform_gemm_k<CG, NBLK, NW>), dim3(n_xform_wg + 8u * (unsigned)seg),
+                       dim3(64 * WAVES), 0, s, M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp,
+                       Tp, Uf, T, chunks, nblk, tiles_n, seg, n_xform_wg, flags, epoch, gave_up,
+                       fused_filter_pauses(n));
+}
+
+// flags: kFusedFlagsPerBoard words per board of the largest batch, zero before the first
+// launch; epoch: a number no earlier launch on these flags has used (grows by one per launch).
+void launch_xform_gemm(half_t* M, const half_t* res, half_t* act_out, half_t* V,
+                       const float* bn_scale, const float* bn_mean, float rfac, int n, int Kp,
+                       int Tp, const half_t* Uf, unsigned long long* flags,
+                       unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
+    if (!xform_gemm_shape(n, Kp, 2)) throw std::invalid_argument("no fused launch for this shape");
+    const int nb = gemm_stream_blocks(n * kTilesPerBoard, Kp);
+    const bool narrow = n * (Kp / 64) <= 64;     // the transform shape launch_out_in_transform takes
+#define LZ_FUSED(CG, NB)                                                                          \
+    launch_xform_gemm_as<CG, NB, 8>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf,   \
+                                    flags, epoch, gave_up, s)
+    if (narrow && nb == 1) LZ_FUSED(16, 1);
+    else if (narrow && nb == 2) LZ_FUSED(16, 2);
+    else if (!narrow && nb == 2) LZ_FUSED(32, 2);
+    else if (!narrow && nb == 4) LZ_FUSED(32, 4);
+    else throw std::invalid_argument("no fused launch instantiated for this batch");
+#undef LZ_FUSED
 }
 
 template <int NK8, int NW>

@@ -533,6 +533,52 @@ def test_graph_replays_match_stream_launches(pkg, netgen, orc):
     plain.close()
 
 
+def test_fused_launches_match_separate_launches(pkg, netgen, orc):
+    """Up to 32 boards an fp16 256-filter tower sends the transform of a layer and the GEMM
+    of the next as one launch when the forward has the device to itself.  Handles that always
+    fuse (LZHIP_FUSE=2), never fuse (0) and decide per forward (the default) must give the
+    same bits, at batches that take each of the fused shapes (one and two 32-row blocks per
+    GEMM work-group with 16-channel transform groups, two and four with 32-channel ones), on
+    one lane and with all lanes busy; and the result agrees with the oracle."""
+    import os
+    import torch
+    print("case: fused launches", flush=True)
+    pipes = {}
+    for mode in ("2", "0", None):
+        if mode is None:
+            os.environ.pop("LZHIP_FUSE", None)
+        else:
+            os.environ["LZHIP_FUSE"] = mode
+        try:
+            net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 4, 256, 3100, pkg.FP16, 32)
+        finally:
+            os.environ.pop("LZHIP_FUSE", None)
+        pipes[mode] = pipe
+    x = netgen.synthetic_inputs(32, seed=3101)
+    for n in (1, 5, 8, 9, 16, 17, 23, 32):
+        want = pipes["0"].forward_batch(x[:n])
+        for mode in ("2", None):
+            got = pipes[mode].forward_batch(x[:n])
+            assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), (n, mode)
+    rp, rv = ref.forward(x[7])
+    want = pipes["0"].forward_batch(x[:16])
+    assert rel_l2(want[0][7], rp) <= 2e-2 and rel_l2(want[1][7], rv) <= 2e-2
+    # every lane at once, many forwards in a row without synchronisation, always fused
+    pipe = pipes["2"]
+    d_in = torch.from_numpy(x).cuda()
+    outs = [(torch.zeros(16, 722, device="cuda"), torch.zeros(16, 361, device="cuda"))
+            for _ in range(pipe.lanes())]
+    torch.cuda.synchronize()
+    for rep in range(8):
+        for k, (pol, val) in enumerate(outs):
+            pipe.forward_batch_device(16, d_in.data_ptr(), pol.data_ptr(), val.data_ptr(), lane=k)
+    pipe.sync()
+    for pol, val in outs:
+        assert np.array_equal(pol.cpu().numpy(), want[0]) and np.array_equal(val.cpu().numpy(), want[1])
+    for pipe in pipes.values():
+        pipe.close()
+
+
 def test_error_behaviour_on_device(pkg, netgen):
     """Calls out of order and arguments out of range are refused with an error code and a
     message, never executed: forward before push_weights, push_weights twice, an even layer
