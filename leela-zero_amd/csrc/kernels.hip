@@ -1477,7 +1477,6 @@ struct StreamWait {
     unsigned long long epoch;
     unsigned* gave_up;     // set to 1 if a wait ran into its spin limit
     int ncg;               // channel groups per board
-    int delay;             // pauses (of ~0.25 us) between the requests of a wavefront's filters
 };
 constexpr int kFlagSpinLimit = 1 << 18;   // polls of ~0.3 us each before a wait gives up
 
@@ -1598,16 +1597,8 @@ __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg,
         // arrive while the transform work-groups are still producing V.  Then wait for the
         // transform work-groups of every board that has a tile among this work-group's rows.
 #pragma unroll
-        for (int kc = 0; kc < NKC; kc++) {
+        for (int kc = 0; kc < NKC; kc++)
             u[kc] = *reinterpret_cast<const int4v*>(Up + (size_t)kc * 64 * 8);
-            if (wait.delay > 0) {
-                // one KiB per wavefront at a time: the transform work-group that shares this
-                // compute unit's memory pipeline is the one everything here waits for
-                __builtin_amdgcn_sched_barrier(0);
-                for (int q = 0; q < wait.delay; q++) __builtin_amdgcn_s_sleep(8);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
         LZ_STAMP(10);
         const int row_lo = blk0 * 32, row_hi = min(blk1 * 32, T);
         const int b_lo = row_lo / kTilesPerBoard, b_hi = (row_hi - 1) / kTilesPerBoard;
@@ -1754,10 +1745,10 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __re
 // after its stores of V -- written through, with the device-scope policy -- have been
 // acknowledged; the GEMM work-groups read V with the same policy.  (Release and acquire
 // fences in their place would write back and invalidate a die's whole L2 once per wavefront:
-// measured 60 us per launch at 16 boards.)  With up to 16 boards both kinds of work-group
-// fit a compute unit together (4 + 8 wavefronts, 168 registers each, 2 x 67 KiB of LDS),
-// so the filters arrive under the transform; with more they follow as the transform's
-// work-groups retire, and the launch still saves the hand-over.
+// measured 60 us per launch at 16 boards.)  With few boards the transform leaves compute
+// units free, and the GEMM work-groups that start there have their filters by the time V
+// is ready; from 16 boards they follow as the transform's work-groups retire, and the
+// launch still saves the hand-over.
 //
 // Waiting is safe because the waiters never hold what the producers need: work-groups are
 // dispatched in the order of their index, so every transform work-group is resident (or
@@ -1776,13 +1767,19 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
     half_t* M, const half_t* res, half_t* act_out, half_t* V, const float* __restrict__ bn_scale,
     const float* __restrict__ bn_mean, float rfac, int n, int Kp, int Tp,
     const half_t* __restrict__ Uf, int T, int chunks, int nblk_total, int tiles_n, int seg,
-    unsigned n_xform_wg, unsigned long long* flags, unsigned long long epoch, unsigned* gave_up,
-    int delay) {
+    unsigned n_xform_wg, unsigned long long* flags, unsigned long long epoch, unsigned* gave_up) {
     typedef BufIO2<half_t>::pair_t pair_t;
     constexpr int NKC = 2 * NW;      // tower layers: as many input as output channels
     constexpr int XBYTES = kPlane * kPlane * (CG / 2) * (int)sizeof(pair_t);
     constexpr int GBYTES = gemm_stream_lds_halves<NKC, NBLK, NW>() * 2;
-    __shared__ __attribute__((aligned(16))) unsigned char lds[XBYTES > GBYTES ? XBYTES : GBYTES];
+    // More than half of a compute unit's 160 KiB, whatever the roles need: two work-groups of
+    // this launch never share a unit.  A GEMM work-group beside a transform work-group sends
+    // its 128 KiB of filters through the memory pipeline that the transform -- which the
+    // whole launch waits for -- is using (measured at 16 boards: 16.7 us per launch with
+    // sharing, also with the filter requests spread out in time, 16.1 without).
+    constexpr int ALONE = 82 * 1024;
+    constexpr int NEED = XBYTES > GBYTES ? XBYTES : GBYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NEED > ALONE ? NEED : ALONE];
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     LZ_STAMP(0);
     if (blockIdx.x < n_xform_wg) {
@@ -1803,7 +1800,7 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
         if (wave >= NW) return;
         wino_gemm_stream_body<NKC, NBLK, NW, true, CG>(
             reinterpret_cast<half_t*>(lds), blockIdx.x - n_xform_wg, V, Uf, M, T, Tp, Kp, chunks,
-            nblk_total, tiles_n, seg, StreamWait{flags, epoch, gave_up, Kp / CG, delay});
+            nblk_total, tiles_n, seg, StreamWait{flags, epoch, gave_up, Kp / CG});
     }
 }
 
@@ -2098,16 +2095,6 @@ bool xform_gemm_shape(int n, int Kp, int elem_bytes) {
     return elem_bytes == 2 && Kp == 256 && n >= 1 && n * (Kp / 64) <= 128;
 }
 
-// Pauses between a GEMM wavefront's 16 filter requests in a fused launch.  Requested all at
-// once, 128 KiB per compute unit go through the memory pipeline that the transform
-// work-group on the same unit is using, and that work-group is what the launch waits for
-// (measured at 16 boards: the slowest transform work-group ends at 10.2 us instead of
-// 8.9, the launch takes 18.1 us instead of 16.6).  Spread out, the filters still arrive
-// before V is ready: two pauses per request from 12 boards (the transform then takes
-// ~9 us), one from 6, none below (its 4 us leave no time to spread anything) and none above
-// 16 boards, where the GEMM work-groups only start when the transform's have left.
-static int fused_filter_pauses(int n) { return n > 16 ? 0 : n >= 12 ? 2 : n >= 6 ? 1 : 0; }
-
 template <int CG, int NBLK, int NW>
 static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, half_t* V,
                                  const float* bn_scale, const float* bn_mean, float rfac, int n,
@@ -2122,8 +2109,7 @@ static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, 
     constexpr int WAVES = NW > fuse_waves(CG) ? NW : fuse_waves(CG);
     hipLaunchKernelGGL((xform_gemm_k<CG, NBLK, NW>), dim3(n_xform_wg + 8u * (unsigned)seg),
                        dim3(64 * WAVES), 0, s, M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp,
-                       Tp, Uf, T, chunks, nblk, tiles_n, seg, n_xform_wg, flags, epoch, gave_up,
-                       fused_filter_pauses(n));
+                       Tp, Uf, T, chunks, nblk, tiles_n, seg, n_xform_wg, flags, epoch, gave_up);
 }
 
 // flags: kFusedFlagsPerBoard words per board of the largest batch, zero before the first
