@@ -834,18 +834,19 @@ private:
             launch_pack_input_bits<P>(d_bits, w.act0, n, kInPlanes, m_C0p, w.stream,
                                       timer(timed, LZHIP_K_PACK));
         launch_in_transform<P>(w.act0, w.V, n, m_C0p, w.Tp, w.stream, timer(timed, LZHIP_K_IN));
-        // Up to 32 boards (fp16, 256 filters) the transform of layer l and the GEMM of layer
-        // l + 1 go out as one launch when this forward has the device to itself: the fused
-        // launch shortens a chain of dependent kernels (one lane: +18 % evaluations/s at one
-        // board, +4..8 % at 4 to 32), but its waiting work-groups hold compute units that
-        // another lane's kernels would otherwise use (three lanes at 8 boards: -20 %).  Both
-        // ways give the same bits.  Not under graph capture (the launch carries a number that
+        // Small batches of fp16 towers (xform_gemm_shape, xform_gemm_pays): the transform of
+        // layer l and the GEMM of layer l + 1 go out as one launch when this forward has the
+        // device to itself: the fused
+        // launch shortens a chain of dependent kernels (one lane, 256 filters: +17 %
+        // evaluations/s at one board, +9 % at 16), but its waiting work-groups hold compute
+        // units that another lane's kernels would otherwise use (three lanes at 8 boards:
+        // -20 %).  Both ways give the same bits.  Not under graph capture (the launch carries a number that
         // has to differ from launch to launch), not when every launch is timed, and not on
         // the static working memory.
         bool fused = false;
         if constexpr (sizeof(P) == 2)
-            fused = m_fuse > 0 && (w.alone || m_fuse > 1) && !timed && !m_use_graph &&
-                    w.flags != nullptr && xform_gemm_shape(n, m_Fp, 2);
+            fused = m_fuse > 0 && ((w.alone && xform_gemm_pays(n, m_Fp)) || m_fuse > 1) && !timed &&
+                    !m_use_graph && w.flags != nullptr && xform_gemm_shape(n, m_Fp, 2);
         int cur = 0, nxt = 1;  // block input (skip) / block output
         launch_gemm<P>(w.V, m_layers[0].U.p, m_layers[0].Uf.p, w.M, Tu, w.Tp, m_layers[0].Cp, m_Fp,
                        w.stream, timer(timed, LZHIP_K_GEMM));

@@ -81,13 +81,15 @@ void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const 
                              hipStream_t s, LaunchTimer* t);
 
 // launch_out_in_transform of one layer and launch_gemm of the next (filters Uf, in the
-// streaming kernel's order) as one launch, for the shapes xform_gemm_shape accepts (fp16,
-// 256 filters, up to 32 boards).  M is read by the transform and rewritten by the GEMM.
+// streaming kernel's order) as one launch, for the shapes xform_gemm_shape accepts (fp16;
+// 256 filters up to 32 boards, 192 up to 42, 128 up to 64).  M is read by the transform and rewritten by the GEMM.
 // flags: kFusedFlagsPerBoard 64-bit words per board (zero before the first launch); epoch: a
 // value no earlier launch on these flags used; *gave_up is set to 1 if a wait inside the
 // launch ran into its limit (the results are then invalid).
 constexpr int kFusedFlagsPerBoard = 16;
 bool xform_gemm_shape(int n, int Kp, int elem_bytes);
+// Whether it is also the faster way for a forward that is alone on the device (measured).
+bool xform_gemm_pays(int n, int Kp);
 void launch_xform_gemm(_Float16* M, const _Float16* res, _Float16* act_out, _Float16* V,
                        const float* bn_scale, const float* bn_mean, float rfac, int n, int Kp,
                        int Tp, const _Float16* Uf, unsigned long long* flags,

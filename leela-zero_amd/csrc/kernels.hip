@@ -2089,10 +2089,22 @@ static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int
     }
 }
 
-// Shapes served by the fused transform + GEMM launch: fp16 towers of 256 filters with the
-// narrow transform shapes (up to 32 boards).
+// Shapes served by the fused transform + GEMM launch: fp16 towers of 128, 192 and 256
+// filters (the widths of the streaming GEMM) at batches that take the narrow transform
+// shapes (up to 32 boards at 256 filters, 42 at 192, 64 at 128).
 bool xform_gemm_shape(int n, int Kp, int elem_bytes) {
-    return elem_bytes == 2 && Kp == 256 && n >= 1 && n * (Kp / 64) <= 128;
+    return elem_bytes == 2 && (Kp == 128 || Kp == 192 || Kp == 256) && n >= 1 &&
+           n * (Kp / 64) <= 128;
+}
+
+// Where the fused launch is the faster way to run a forward that has the device to itself
+// (one lane, 40x256 / 15x192 / 10x128, evaluations per second against separate launches):
+// 256 filters +17 % at 1 board, +8 % at 4, 0 at 8, +9 % at 16 and 20, +7 % at 24, 0 at 32;
+// 192 filters -2..+2 % up to 8 boards, +3..+6 % from 12 to 42; 128 filters -1..-8 % up to
+// 20 boards, +2..+6 % from 24 to 64.  (What it saves is the hand-over between two launches
+// and, with few boards, the wait for the filters: a quarter as many bytes at 128 filters.)
+bool xform_gemm_pays(int n, int Kp) {
+    return Kp == 256 || (Kp == 192 && n >= 12) || (Kp == 128 && n >= 24);
 }
 
 template <int CG, int NBLK, int NW>
@@ -2112,6 +2124,28 @@ static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, 
                        Tp, Uf, T, chunks, nblk, tiles_n, seg, n_xform_wg, flags, epoch, gave_up);
 }
 
+template <int NW>
+static void launch_xform_gemm_nw(half_t* M, const half_t* res, half_t* act_out, half_t* V,
+                                 const float* bn_scale, const float* bn_mean, float rfac, int n,
+                                 int Kp, int Tp, const half_t* Uf, unsigned long long* flags,
+                                 unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
+    const int nb = gemm_stream_blocks(n * kTilesPerBoard, Kp);
+    const bool narrow = n * (Kp / 64) <= 64;     // the transform shape launch_out_in_transform takes
+#define LZ_FUSED(CG, NB)                                                                          \
+    launch_xform_gemm_as<CG, NB, NW>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf,  \
+                                     flags, epoch, gave_up, s)
+    // the pairs that occur: 16-channel groups up to 64 / (Kp / 64) boards, i.e. up to 7, 14 or
+    // (128 filters) 25 blocks of 32 rows per position; 32-channel groups up to twice that
+    if (narrow && nb == 1) LZ_FUSED(16, 1);
+    else if (narrow && nb == 2) LZ_FUSED(16, 2);
+    else if (narrow && nb == 4) LZ_FUSED(16, 4);
+    else if (!narrow && nb == 2) LZ_FUSED(32, 2);
+    else if (!narrow && nb == 4) LZ_FUSED(32, 4);
+    else if (!narrow && nb == 8) LZ_FUSED(32, 8);
+    else throw std::invalid_argument("no fused launch instantiated for this batch");
+#undef LZ_FUSED
+}
+
 // flags: kFusedFlagsPerBoard words per board of the largest batch, zero before the first
 // launch; epoch: a number no earlier launch on these flags has used (grows by one per launch).
 void launch_xform_gemm(half_t* M, const half_t* res, half_t* act_out, half_t* V,
@@ -2119,17 +2153,11 @@ void launch_xform_gemm(half_t* M, const half_t* res, half_t* act_out, half_t* V,
                        int Tp, const half_t* Uf, unsigned long long* flags,
                        unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
     if (!xform_gemm_shape(n, Kp, 2)) throw std::invalid_argument("no fused launch for this shape");
-    const int nb = gemm_stream_blocks(n * kTilesPerBoard, Kp);
-    const bool narrow = n * (Kp / 64) <= 64;     // the transform shape launch_out_in_transform takes
-#define LZ_FUSED(CG, NB)                                                                          \
-    launch_xform_gemm_as<CG, NB, 8>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf,   \
-                                    flags, epoch, gave_up, s)
-    if (narrow && nb == 1) LZ_FUSED(16, 1);
-    else if (narrow && nb == 2) LZ_FUSED(16, 2);
-    else if (!narrow && nb == 2) LZ_FUSED(32, 2);
-    else if (!narrow && nb == 4) LZ_FUSED(32, 4);
-    else throw std::invalid_argument("no fused launch instantiated for this batch");
-#undef LZ_FUSED
+    switch (Kp) {
+        case 256: launch_xform_gemm_nw<8>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s); break;
+        case 192: launch_xform_gemm_nw<6>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s); break;
+        default: launch_xform_gemm_nw<4>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s); break;
+    }
 }
 
 template <int NK8, int NW>

@@ -533,16 +533,22 @@ def test_graph_replays_match_stream_launches(pkg, netgen, orc):
     plain.close()
 
 
-def test_fused_launches_match_separate_launches(pkg, netgen, orc):
-    """Up to 32 boards an fp16 256-filter tower sends the transform of a layer and the GEMM
-    of the next as one launch when the forward has the device to itself.  Handles that always
-    fuse (LZHIP_FUSE=2), never fuse (0) and decide per forward (the default) must give the
-    same bits, at batches that take each of the fused shapes (one and two 32-row blocks per
-    GEMM work-group with 16-channel transform groups, two and four with 32-channel ones), on
-    one lane and with all lanes busy; and the result agrees with the oracle."""
+@pytest.mark.parametrize("filters,maxb,batches", [
+    (256, 32, (1, 5, 8, 9, 16, 17, 23, 32)),
+    (192, 42, (1, 7, 10, 15, 21, 22, 37, 42)),
+    (128, 64, (1, 8, 9, 18, 32, 33, 36, 64)),
+])
+def test_fused_launches_match_separate_launches(pkg, netgen, orc, filters, maxb, batches):
+    """An fp16 tower of 128, 192 or 256 filters sends the transform of a layer and the GEMM of
+    the next as one launch when the forward has the device to itself, up to the batch where
+    the transform changes to its 64-channel shape.  Handles that always fuse (LZHIP_FUSE=2),
+    never fuse (0) and decide per forward (the default) must give the same bits, at batches
+    that take each of the fused shapes (1, 2, 4 or 8 blocks of 32 rows per GEMM work-group,
+    16- or 32-channel transform groups), on one lane and with all lanes busy; and the result
+    agrees with the oracle."""
     import os
     import torch
-    print("case: fused launches", flush=True)
+    print("case: fused launches, %d filters" % filters, flush=True)
     pipes = {}
     for mode in ("2", "0", None):
         if mode is None:
@@ -550,28 +556,29 @@ def test_fused_launches_match_separate_launches(pkg, netgen, orc):
         else:
             os.environ["LZHIP_FUSE"] = mode
         try:
-            net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 4, 256, 3100, pkg.FP16, 32)
+            net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 4, filters, 3100, pkg.FP16, maxb)
         finally:
             os.environ.pop("LZHIP_FUSE", None)
         pipes[mode] = pipe
-    x = netgen.synthetic_inputs(32, seed=3101)
-    for n in (1, 5, 8, 9, 16, 17, 23, 32):
+    x = netgen.synthetic_inputs(maxb, seed=3101)
+    for n in batches:
         want = pipes["0"].forward_batch(x[:n])
         for mode in ("2", None):
             got = pipes[mode].forward_batch(x[:n])
             assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), (n, mode)
     rp, rv = ref.forward(x[7])
-    want = pipes["0"].forward_batch(x[:16])
+    nb = batches[4]
+    want = pipes["0"].forward_batch(x[:nb])
     assert rel_l2(want[0][7], rp) <= 2e-2 and rel_l2(want[1][7], rv) <= 2e-2
     # every lane at once, many forwards in a row without synchronisation, always fused
     pipe = pipes["2"]
     d_in = torch.from_numpy(x).cuda()
-    outs = [(torch.zeros(16, 722, device="cuda"), torch.zeros(16, 361, device="cuda"))
+    outs = [(torch.zeros(nb, 722, device="cuda"), torch.zeros(nb, 361, device="cuda"))
             for _ in range(pipe.lanes())]
     torch.cuda.synchronize()
     for rep in range(8):
         for k, (pol, val) in enumerate(outs):
-            pipe.forward_batch_device(16, d_in.data_ptr(), pol.data_ptr(), val.data_ptr(), lane=k)
+            pipe.forward_batch_device(nb, d_in.data_ptr(), pol.data_ptr(), val.data_ptr(), lane=k)
     pipe.sync()
     for pol, val in outs:
         assert np.array_equal(pol.cpu().numpy(), want[0]) and np.array_equal(val.cpu().numpy(), want[1])
