@@ -192,6 +192,7 @@ public:
         *m_gave_up.p = 0;
         // measurement knob: 0 never, 1 when the forward is alone on the device, 2 always
         if (const char* e = std::getenv("LZHIP_FUSE")) m_fuse = std::atoi(e);
+        if (const char* e = std::getenv("LZHIP_INPLACE")) m_in_place = std::atoi(e) != 0;
         m_scalar.alloc(4);
         for (int i = 0; i < kTimerPool; i++) {
             HIP_CHECK(hipEventCreate(&m_ev_start[i]));
@@ -847,6 +848,14 @@ private:
         if constexpr (sizeof(P) == 2)
             fused = m_fuse > 0 && ((w.alone && xform_gemm_pays(n, m_Fp)) || m_fuse > 1) && !timed &&
                     !m_use_graph && w.flags != nullptr && xform_gemm_shape(n, m_Fp, 2);
+        // With the streaming GEMM the tower's layers work in place: M_l is written over V_l
+        // and V_{l+1} over M_l (see the kernels), so a lane's tiles are one array instead of
+        // two and the lanes' working sets (2 or 3 x 33 MB of tiles less at 64 boards) fit the
+        // 256 MB memory-side cache.  Layer 0 reads 64 padded planes and keeps its own output.
+        P* tiles = w.M;
+        const bool in_place = m_in_place && !fused && m_layers.size() > 1 &&
+                              gemm_stream_shape(Tu, m_Fp, m_Fp, (int)sizeof(P)) &&
+                              m_layers[1].Uf.p != nullptr;
         int cur = 0, nxt = 1;  // block input (skip) / block output
         launch_gemm<P>(w.V, m_layers[0].U.p, m_layers[0].Uf.p, w.M, Tu, w.Tp, m_layers[0].Cp, m_Fp,
                        w.stream, timer(timed, LZHIP_K_GEMM));
@@ -856,7 +865,7 @@ private:
             const P* res = (block_end && l >= 2) ? w.act[cur] : nullptr;
             P* out = l == 0 ? w.act[cur] : w.act[nxt];
             if (l == nl - 1) {
-                launch_out_transform<P>(w.M, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp,
+                launch_out_transform<P>(tiles, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp,
                                         w.Tp, w.stream, timer(timed, LZHIP_K_OUT));
                 launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, w.stream,
                                     timer(timed, LZHIP_K_HEAD));
@@ -872,10 +881,11 @@ private:
                     }
                 }
                 if (!done) {
-                    launch_out_in_transform<P>(w.M, res, block_end ? out : nullptr, w.V,
+                    launch_out_in_transform<P>(tiles, res, block_end ? out : nullptr, w.V,
                                                L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, w.Tp,
                                                w.stream, timer(timed, LZHIP_K_OUTIN));
-                    launch_gemm<P>(w.V, N.U.p, N.Uf.p, w.M, Tu, w.Tp, N.Cp, m_Fp, w.stream,
+                    if (in_place) tiles = w.V;
+                    launch_gemm<P>(w.V, N.U.p, N.Uf.p, tiles, Tu, w.Tp, N.Cp, m_Fp, w.stream,
                                    timer(timed, LZHIP_K_GEMM));
                 }
             }
@@ -996,6 +1006,7 @@ private:
     LaunchTimer m_timer;
     bool m_use_graph = std::getenv("LZHIP_GRAPH") != nullptr;
     int m_fuse = 1;                      // fused transform + GEMM launches (see enqueue_forward)
+    bool m_in_place = true;              // tower layers keep V and M in one array (see enqueue_forward)
     PinnedBuf<unsigned> m_gave_up;       // set by a fused launch whose wait ran into its limit
 };
 

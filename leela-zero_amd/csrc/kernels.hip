@@ -681,11 +681,13 @@ __device__ __forceinline__ int out_in_transform_body(
     return item;
 }
 
+// M and Vn may be one array (every value of M is in a register before the same lane writes
+// the value of V that takes its place), so neither is declared free of aliases.
 template <typename P, int CG>
 __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
-    const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ act_out,
-    P* __restrict__ Vn, const float* __restrict__ bn_scale, const float* __restrict__ bn_mean,
-    float rfac, int n, int Kp, int Tp) {
+    const P* M, const P* __restrict__ res, P* __restrict__ act_out, P* Vn,
+    const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int n,
+    int Kp, int Tp) {
     __shared__ typename BufIO2<P>::pair_t ybuf[kPlane * kPlane * (CG / 2)];
     (void)out_in_transform_body<P, CG, xform_store_policy<CG>()>(ybuf, blockIdx.x, M, res, act_out, Vn, bn_scale, bn_mean,
                                        rfac, n, Kp, Tp);
@@ -1722,10 +1724,13 @@ __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg,
     send_rows(NBLK - 1);
 }
 
+// V and M may be one array when the tile is the whole row of M (tiles_n == 1, as many input
+// as output channels): a work-group has a block of V in LDS before it writes the block of M
+// that takes its place, and no other work-group touches those rows.
 template <int NKC, int NBLK, int NW>
-__global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* __restrict__ V,
+__global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* V,
                                                           const half_t* __restrict__ Uf,
-                                                          half_t* __restrict__ M, int T, int Tp,
+                                                          half_t* M, int T, int Tp,
                                                           int Kp, int chunks, int nblk_total,
                                                           int tiles_n, int seg) {
     __shared__ __attribute__((aligned(16))) half_t smem[gemm_stream_lds_halves<NKC, NBLK, NW>()];
@@ -1822,9 +1827,9 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
 // U_p[32 wb + gemm_stream_channel(l % 32)][8 j + 4 (l / 32) + 0..3].
 
 template <int NK8, int NBLK, int NW>
-__global__ __launch_bounds__(64 * NW) void wino_gemm_stream32_k(const float* __restrict__ V,
+__global__ __launch_bounds__(64 * NW) void wino_gemm_stream32_k(const float* V,   // may be M
                                                                 const float* __restrict__ Uf,
-                                                                float* __restrict__ M, int T,
+                                                                float* M, int T,
                                                                 int Tp, int Kp, int chunks,
                                                                 int nblk_total, int seg) {
     constexpr int D = kStreamAhead;
