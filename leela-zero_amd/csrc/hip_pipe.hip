@@ -190,7 +190,8 @@ public:
         }
         m_gave_up.alloc(1);
         *m_gave_up.p = 0;
-        // measurement knob: 0 never, 1 when the forward is alone on the device, 2 always
+        // measurement knob: 0 never, 1 where it pays and the forward is alone on the device,
+        // 2 always (one array), 3 always (two arrays, up to 8 boards)
         if (const char* e = std::getenv("LZHIP_FUSE")) m_fuse = std::atoi(e);
         if (const char* e = std::getenv("LZHIP_INPLACE")) m_in_place = std::atoi(e) != 0;
         m_scalar.alloc(4);
@@ -835,19 +836,22 @@ private:
             launch_pack_input_bits<P>(d_bits, w.act0, n, kInPlanes, m_C0p, w.stream,
                                       timer(timed, LZHIP_K_PACK));
         launch_in_transform<P>(w.act0, w.V, n, m_C0p, w.Tp, w.stream, timer(timed, LZHIP_K_IN));
-        // Small batches of fp16 towers (xform_gemm_shape, xform_gemm_pays): the transform of
-        // layer l and the GEMM of layer l + 1 go out as one launch when this forward has the
-        // device to itself: the fused
+        // Small batches of fp16 towers (xform_gemm_shape; xform_gemm_pays says which of the
+        // launch's two forms, if any): the transform of layer l and the GEMM of layer l + 1 go
+        // out as one launch when this forward has the device to itself: the fused
         // launch shortens a chain of dependent kernels (one lane, 256 filters: +17 %
         // evaluations/s at one board, +9 % at 16), but its waiting work-groups hold compute
         // units that another lane's kernels would otherwise use (three lanes at 8 boards:
         // -20 %).  Both ways give the same bits.  Not under graph capture (the launch carries a number that
         // has to differ from launch to launch), not when every launch is timed, and not on
         // the static working memory.
-        bool fused = false;
-        if constexpr (sizeof(P) == 2)
-            fused = m_fuse > 0 && ((w.alone && xform_gemm_pays(n, m_Fp)) || m_fuse > 1) && !timed &&
-                    !m_use_graph && w.flags != nullptr && xform_gemm_shape(n, m_Fp, 2);
+        bool fused = false, fused_two_arrays = false;
+        if constexpr (sizeof(P) == 2) {
+            const int form = m_fuse == 2 ? 1 : m_fuse == 3 ? 2 : xform_gemm_pays(n, m_Fp);
+            fused = m_fuse > 0 && form > 0 && (w.alone || m_fuse > 1) && !timed && !m_use_graph &&
+                    w.flags != nullptr && xform_gemm_shape(n, m_Fp, 2) && (form == 1 || n <= 8);
+            fused_two_arrays = form == 2;
+        }
         // With the streaming GEMM the tower's layers work in place: M_l is written over V_l
         // and V_{l+1} over M_l (see the kernels), so a lane's tiles are one array instead of
         // two and the lanes' working sets (2 or 3 x 33 MB of tiles less at 64 boards) fit the
@@ -874,7 +878,8 @@ private:
                 bool done = false;
                 if constexpr (sizeof(P) == 2) {
                     if (fused) {
-                        launch_xform_gemm(w.M, res, block_end ? out : nullptr, w.V, L.d_scale.p,
+                        launch_xform_gemm(w.M, res, block_end ? out : nullptr,
+                                          fused_two_arrays ? w.V : w.M, L.d_scale.p,
                                           L.d_mean.p, L.rfac, n, m_Fp, w.Tp, N.Uf.p, w.flags,
                                           ++*w.epoch, m_gave_up.p, w.stream);
                         done = true;

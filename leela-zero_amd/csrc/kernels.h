@@ -88,8 +88,9 @@ void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const 
 // launch ran into its limit (the results are then invalid).
 constexpr int kFusedFlagsPerBoard = 16;
 bool xform_gemm_shape(int n, int Kp, int elem_bytes);
-// Whether it is also the faster way for a forward that is alone on the device (measured).
-bool xform_gemm_pays(int n, int Kp);
+// Which form is the faster way for a forward that is alone on the device (measured): 0 none,
+// 1 V and M one array (launch_xform_gemm with V == M), 2 two arrays (V != M, up to 8 boards).
+int xform_gemm_pays(int n, int Kp);
 void launch_xform_gemm(_Float16* M, const _Float16* res, _Float16* act_out, _Float16* V,
                        const float* bn_scale, const float* bn_mean, float rfac, int n, int Kp,
                        int Tp, const _Float16* Uf, unsigned long long* flags,

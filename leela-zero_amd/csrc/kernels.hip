@@ -1761,13 +1761,16 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* V,
 // nothing.  A wait is bounded all the same: after kFlagSpinLimit polls it reports through
 // `gave_up` and goes on, so that the launch always ends.
 //
-// Inside such a launch V is laid out channel group by channel group ([36][Kp / CG][Tp][CG],
-// see out_in_transform_body): nothing outside the launch reads it.
-//
 // The buffers: the transform reads M and writes V, the GEMM reads V and writes M -- the
 // same M.  A GEMM work-group writes rows of M only after every transform work-group of
-// the boards those rows belong to has finished, i.e. after their last read.
-template <int CG, int NBLK, int NW>
+// the boards those rows belong to has finished, i.e. after their last read.  Two forms:
+//   SLABV = false: V and M are one array in M's layout, each stage overwriting its input
+//     (as the separate launches do); the written-through 32- and 64-byte pieces of V then
+//     land in lines this die's L2 already holds.  The form for 14 boards and more.
+//   SLABV = true: V is a second array, laid out channel group by channel group
+//     ([36][Kp / CG][Tp][CG], see out_in_transform_body; nothing outside the launch reads
+//     it), so that the transform writes whole lines.  The faster form at 1 to 6 boards.
+template <int CG, int NBLK, int NW, bool SLABV>
 __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) void xform_gemm_k(
     half_t* M, const half_t* res, half_t* act_out, half_t* V, const float* __restrict__ bn_scale,
     const float* __restrict__ bn_mean, float rfac, int n, int Kp, int Tp,
@@ -1789,7 +1792,7 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
     LZ_STAMP(0);
     if (blockIdx.x < n_xform_wg) {
         if (wave >= fuse_waves(CG)) return;    // the block is sized for the larger role
-        const int item = out_in_transform_body<half_t, CG, kStoreThrough, true>(
+        const int item = out_in_transform_body<half_t, CG, kStoreThrough, SLABV>(
             reinterpret_cast<pair_t*>(lds), blockIdx.x, M, res, act_out, V, bn_scale, bn_mean,
             rfac, n, Kp, Tp);
         if (item < 0) return;                  // uniform over the work-group
@@ -1803,7 +1806,7 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
         LZ_STAMP(7);
     } else {
         if (wave >= NW) return;
-        wino_gemm_stream_body<NKC, NBLK, NW, true, CG>(
+        wino_gemm_stream_body<NKC, NBLK, NW, true, SLABV ? CG : 0>(
             reinterpret_cast<half_t*>(lds), blockIdx.x - n_xform_wg, V, Uf, M, T, Tp, Kp, chunks,
             nblk_total, tiles_n, seg, StreamWait{flags, epoch, gave_up, Kp / CG});
     }
@@ -2102,17 +2105,28 @@ bool xform_gemm_shape(int n, int Kp, int elem_bytes) {
            n * (Kp / 64) <= 128;
 }
 
-// Where the fused launch is the faster way to run a forward that has the device to itself
-// (one lane, 40x256 / 15x192 / 10x128, evaluations per second against separate launches):
-// 256 filters +17 % at 1 board, +8 % at 4, 0 at 8, +9 % at 16 and 20, +7 % at 24, 0 at 32;
-// 192 filters -2..+2 % up to 8 boards, +3..+6 % from 12 to 42; 128 filters -1..-8 % up to
-// 20 boards, +2..+6 % from 24 to 64.  (What it saves is the hand-over between two launches
-// and, with few boards, the wait for the filters: a quarter as many bytes at 128 filters.)
-bool xform_gemm_pays(int n, int Kp) {
-    return Kp == 256 || (Kp == 192 && n >= 12) || (Kp == 128 && n >= 24);
+// Which form of the fused launch, if any, is the faster way to run a forward that has the
+// device to itself: 0 none (separate launches), 1 one array, 2 two arrays.  Measured on one
+// lane (40x256 / 15x192 / 10x128, evaluations per second against separate launches, which
+// also work in place):
+//   256 filters  two arrays +17 % at 1 board, +9 % at 2, +6 % at 4, +3 % at 6 (one array
+//                +10, +9, +3, +3 %), both -4..-7 % at 8; one array -1..-3 % at 10 to 14,
+//                +8 % at 16, +5 % at 20, +9 % at 24, +3 % at 32
+//   192 filters  neither form up to 20 boards (-3..-11 %); one array +7 % at 24, +10 % at
+//                32, +19 % at 42
+//   128 filters  neither form up to 24 boards (-3..-12 %); one array +5 % at 32, +3 % at
+//                42, +8 % at 48, +25 % at 64
+// The one-array form pays where the transform's work-groups fill the device, so that GEMM
+// work-groups start as those retire instead of after a hand-over between launches; the
+// two-array form where a few boards leave most of the device to GEMM work-groups that fetch
+// their filters (128 KiB each at 256 filters) while the transform runs.
+int xform_gemm_pays(int n, int Kp) {
+    if (Kp == 256) return n <= 6 ? 2 : n >= 16 ? 1 : 0;
+    if (Kp == 192) return n >= 22 ? 1 : 0;
+    return n >= 32 ? 1 : 0;
 }
 
-template <int CG, int NBLK, int NW>
+template <int CG, int NBLK, int NW, bool SLABV>
 static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, half_t* V,
                                  const float* bn_scale, const float* bn_mean, float rfac, int n,
                                  int Kp, int Tp, const half_t* Uf, unsigned long long* flags,
@@ -2124,9 +2138,10 @@ static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, 
     const int seg = (kPos * chunks * tiles_n + 7) / 8;
     const unsigned n_xform_wg = 8u * (unsigned)((n * (Kp / CG) + 7) / 8);
     constexpr int WAVES = NW > fuse_waves(CG) ? NW : fuse_waves(CG);
-    hipLaunchKernelGGL((xform_gemm_k<CG, NBLK, NW>), dim3(n_xform_wg + 8u * (unsigned)seg),
-                       dim3(64 * WAVES), 0, s, M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp,
-                       Tp, Uf, T, chunks, nblk, tiles_n, seg, n_xform_wg, flags, epoch, gave_up);
+    hipLaunchKernelGGL((xform_gemm_k<CG, NBLK, NW, SLABV>),
+                       dim3(n_xform_wg + 8u * (unsigned)seg), dim3(64 * WAVES), 0, s, M, res,
+                       act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, T, chunks, nblk, tiles_n,
+                       seg, n_xform_wg, flags, epoch, gave_up);
 }
 
 template <int NW>
@@ -2136,21 +2151,27 @@ static void launch_xform_gemm_nw(half_t* M, const half_t* res, half_t* act_out, 
                                  unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
     const int nb = gemm_stream_blocks(n * kTilesPerBoard, Kp);
     const bool narrow = n * (Kp / 64) <= 64;     // the transform shape launch_out_in_transform takes
-#define LZ_FUSED(CG, NB)                                                                          \
-    launch_xform_gemm_as<CG, NB, NW>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf,  \
-                                     flags, epoch, gave_up, s)
+#define LZ_FUSED(CG, NB, SLABV)                                                                   \
+    launch_xform_gemm_as<CG, NB, NW, SLABV>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp,   \
+                                            Tp, Uf, flags, epoch, gave_up, s)
+    if (V != M) {   // the second array: the few-board form
+        if (narrow && nb == 1) LZ_FUSED(16, 1, true);
+        else throw std::invalid_argument("the two-array fused launch serves up to 8 boards");
+        return;
+    }
     // the pairs that occur: 16-channel groups up to 64 / (Kp / 64) boards, i.e. up to 7, 14 or
     // (128 filters) 25 blocks of 32 rows per position; 32-channel groups up to twice that
-    if (narrow && nb == 1) LZ_FUSED(16, 1);
-    else if (narrow && nb == 2) LZ_FUSED(16, 2);
-    else if (narrow && nb == 4) LZ_FUSED(16, 4);
-    else if (!narrow && nb == 2) LZ_FUSED(32, 2);
-    else if (!narrow && nb == 4) LZ_FUSED(32, 4);
-    else if (!narrow && nb == 8) LZ_FUSED(32, 8);
+    if (narrow && nb == 1) LZ_FUSED(16, 1, false);
+    else if (narrow && nb == 2) LZ_FUSED(16, 2, false);
+    else if (narrow && nb == 4) LZ_FUSED(16, 4, false);
+    else if (!narrow && nb == 2) LZ_FUSED(32, 2, false);
+    else if (!narrow && nb == 4) LZ_FUSED(32, 4, false);
+    else if (!narrow && nb == 8) LZ_FUSED(32, 8, false);
     else throw std::invalid_argument("no fused launch instantiated for this batch");
 #undef LZ_FUSED
 }
 
+// V == M: the one-array form; V != M: the two-array form (up to 8 boards).
 // flags: kFusedFlagsPerBoard words per board of the largest batch, zero before the first
 // launch; epoch: a number no earlier launch on these flags has used (grows by one per launch).
 void launch_xform_gemm(half_t* M, const half_t* res, half_t* act_out, half_t* V,

@@ -540,9 +540,10 @@ def test_graph_replays_match_stream_launches(pkg, netgen, orc):
 ])
 def test_fused_launches_match_separate_launches(pkg, netgen, orc, filters, maxb, batches):
     """An fp16 tower of 128, 192 or 256 filters sends the transform of a layer and the GEMM of
-    the next as one launch when the forward has the device to itself, up to the batch where
-    the transform changes to its 64-channel shape.  Handles that always fuse (LZHIP_FUSE=2),
-    never fuse (0) and decide per forward (the default) must give the same bits, at batches
+    the next as one launch where that is faster and the forward has the device to itself, up
+    to the batch where the transform changes to its 64-channel shape.  Handles that always fuse
+    with V and M in one array (LZHIP_FUSE=2), that fuse with two arrays up to 8 boards (3),
+    that never fuse (0) and that decide per forward (the default) must give the same bits, at batches
     that take each of the fused shapes (1, 2, 4 or 8 blocks of 32 rows per GEMM work-group,
     16- or 32-channel transform groups), on one lane and with all lanes busy; and the result
     agrees with the oracle."""
@@ -550,7 +551,7 @@ def test_fused_launches_match_separate_launches(pkg, netgen, orc, filters, maxb,
     import torch
     print("case: fused launches, %d filters" % filters, flush=True)
     pipes = {}
-    for mode in ("2", "0", None):
+    for mode in ("2", "3", "0", None):
         if mode is None:
             os.environ.pop("LZHIP_FUSE", None)
         else:
@@ -563,7 +564,7 @@ def test_fused_launches_match_separate_launches(pkg, netgen, orc, filters, maxb,
     x = netgen.synthetic_inputs(maxb, seed=3101)
     for n in batches:
         want = pipes["0"].forward_batch(x[:n])
-        for mode in ("2", None):
+        for mode in ("2", "3", None):
             got = pipes[mode].forward_batch(x[:n])
             assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), (n, mode)
     rp, rv = ref.forward(x[7])
