@@ -697,16 +697,17 @@ template <typename P>
 void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
                              const float* bn_mean, float rfac, int n, int Kp, int Tp,
                              hipStream_t s, LaunchTimer* t) {
-    // The narrowest shape whose work-groups fit the 256 compute units in one go: a board's
-    // arithmetic then spreads over the most units (measured at 256 filters, per launch:
-    // 16 channels 7.7 us against 8.4 with 32 and 9.7 with 64 at batch 16; 32 channels 10.1
-    // against 10.4 with 64 and 11.0 with 16 at batch 32; 64 channels from batch 33: 10.5
-    // against 13.0 at 36).  The narrow shapes only pay with the die-aware item order of the
-    // kernel: dealt round-robin over the dies, their work-groups fetch every line of M once
-    // per die that holds a piece of it (16 channels at batch 16: 11.2 us).
+    // With few boards a narrow shape spreads a board's arithmetic over more compute units;
+    // the 64-channel shape moves whole lines.  Measured at 256 filters with the layers working
+    // in place (transform + GEMM per layer, us, with 16 / 32 / 64 channels per work-group):
+    // 8 boards 11.7 / 12.8 / 14.0, 16 boards 14.6 / 15.3 / 15.4, 20 boards 17.3 / 16.5 / 16.6,
+    // 24 boards 18.4 / 17.5 / 16.8, 32 boards 21.9 / 20.5 / 19.9, 40 boards 24.7 / 24.8 / 20.8.
+    // The narrow shapes only pay with the die-aware item order of the kernel: dealt round-robin
+    // over the dies, their work-groups fetch every line of M once per die that holds a piece
+    // of it (16 channels at batch 16: 11.2 us per launch against 7.7).
     const int items64 = n * (Kp / 64);
     auto grid = [](int items) { return dim3((unsigned)(8 * ((items + 7) / 8))); };
-    if (items64 > 128)
+    if (items64 > 80)
         launch(out_in_transform_k<P, 64>, grid(items64), dim3(fuse_waves(64) * 64), s, t, M, res,
                act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
     else if (items64 > 64)
@@ -2150,7 +2151,7 @@ static void launch_xform_gemm_nw(half_t* M, const half_t* res, half_t* act_out, 
                                  int Kp, int Tp, const half_t* Uf, unsigned long long* flags,
                                  unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
     const int nb = gemm_stream_blocks(n * kTilesPerBoard, Kp);
-    const bool narrow = n * (Kp / 64) <= 64;     // the transform shape launch_out_in_transform takes
+    const bool narrow = n * (Kp / 64) <= 64;     // 16-channel transform groups, else 32
 #define LZ_FUSED(CG, NB, SLABV)                                                                   \
     launch_xform_gemm_as<CG, NB, NW, SLABV>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp,   \
                                             Tp, Uf, flags, epoch, gave_up, s)

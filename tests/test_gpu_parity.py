@@ -165,7 +165,7 @@ def test_forward_parity_wide_batches(pkg, netgen, orc, precision, batch):
     the streaming kernel with 1, 2, 4, 8 and 16 blocks of 32 tile rows per work-group, which
     change at 9, 18, 36 and 72 boards; fp32:
     256x256 tiles from 41 boards, 128x128 from 21, 128x64 with padded rows below; fused
-    transform: 64 channels per work-group from 33 boards, 32 from 17, 16 below), in both
+    transform: 64 channels per work-group from 21 boards, 32 from 17, 16 below), in both
     precisions, including batches whose tile count is not a multiple of any tile height."""
     print("case: wide 3x256 b%d precision=%d" % (batch, precision), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 256, 3000, precision, batch)
