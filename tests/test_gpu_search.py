@@ -184,6 +184,44 @@ def test_selfplay_with_device_heads(pkg, netgen, orc):
     pipe.close()
 
 
+def test_timed_evaluations_and_process_counters(pkg, netgen):
+    """lzhip_timed_evaluations (events around copy-in + tower + device heads + copy-out)
+    returns what lzhip_evaluate_batch returns for the same batch, and a positive time that
+    grows with the number of repetitions; the process-wide batch counters (the engine's
+    batch_stats) count this process's queued batches: singles + multiples = batches,
+    positions and slots grow by what one handle's own statistics say."""
+    print("case: timed evaluations", flush=True)
+    net = netgen.make_network(2, 64, 5)
+    w, h = netgen.prepare(net)
+    pipe = pkg.HIPScheduler(pkg.FP16, 8)
+    pipe.initialize(64)
+    pipe.push_weights(6, 18, 64, w)
+    x = netgen.synthetic_inputs(8, seed=3)
+    with pytest.raises(ValueError):
+        pipe.timed_evaluations(x, 2)               # heads not pushed
+    pipe.push_heads(h)
+    policy, value, _ = pipe.evaluate_batch(x)
+    ms3, p3, v3 = pipe.timed_evaluations(x, 3)
+    ms30, p30, v30 = pipe.timed_evaluations(x, 30)
+    assert np.array_equal(p3, policy) and np.array_equal(v3, value)
+    assert np.array_equal(p30, policy) and np.array_equal(v30, value)
+    assert 0.0 < ms3 < ms30 < 1000.0
+    with pytest.raises(ValueError):
+        pipe.timed_evaluations(x, 0)
+    before = pkg.process_batch_stats()
+    pipe.reset_stats()
+    for i in range(5):
+        pipe.forward(x[i])
+    st, after = pipe.stats(), pkg.process_batch_stats()
+    assert st["requests"] == 5
+    assert (after["single_evals"] + after["batch_evals"]
+            - before["single_evals"] - before["batch_evals"]) == st["batches"]
+    assert after["positions"] - before["positions"] == st["requests"]
+    assert after["slots"] - before["slots"] == st["batch_slots"]
+    assert after["single_evals"] - before["single_evals"] == 5      # one caller: batches of one
+    pipe.close()
+
+
 def test_selfplay_argument_checks(pkg, netgen, orc):
     print("case: selfplay argument checks", flush=True)
     pipe, h, ref, h_ref = make(pkg, netgen, orc, 1, 64, 2, 0, 2)
