@@ -7,6 +7,7 @@
 
 #include <cstdlib>
 #include <stdexcept>
+#include <type_traits>
 
 #include <hip/hip_ext.h>
 
@@ -2409,68 +2410,68 @@ void head_fc_fragments(const float* W, bool policy, float* dst) {
                     }
 }
 
-__global__ __launch_bounds__(256) void heads_fc_k(const float* __restrict__ pol,
-                                                  const float* __restrict__ val, HeadParams hp,
-                                                  float* __restrict__ logits,
-                                                  float* __restrict__ hidden, int n) {
-    constexpr int ROW = kHeadKPad + 1;   // odd row length: conflict-free column reads
-    __shared__ float xs[32 * ROW];
-    const int tasks = kHeadColsPol + kHeadColsVal;
-    const int rb = blockIdx.x / tasks, task = blockIdx.x - rb * tasks;
-    const bool policy = task < kHeadColsPol;
-    const int cb = policy ? task : task - kHeadColsPol;
-    const int K = policy ? 2 * kPts : kPts;
-    const int steps = policy ? kHeadStepsPol : kHeadStepsVal;
-    const int kpad = 4 * steps * 2;
+// One layer's share of heads_fc_k.  Everything a work-group reads has been out of the caches
+// since the last call (a tower of 81 layers ran in between) and the planes have just been
+// written on other dies, so a round trip to memory takes ~2 us here: the wavefront's whole
+// share of the weights (23 or 12 KiB) and, per thread, its 92 or 48 values of the planes are
+// requested before the first is used.
+template <bool POL>
+__device__ __forceinline__ void heads_fc_body(float* xs, const float* __restrict__ src,
+                                              const HeadParams& hp, float* __restrict__ out,
+                                              int cb, int r0, int n) {
+    constexpr int STEPS = POL ? kHeadStepsPol : kHeadStepsVal;
+    constexpr int G = STEPS / 4;             // 16-byte weight loads per lane
+    constexpr int KP = 4 * STEPS * 2;        // padded contraction length
+    constexpr int KK = POL ? 2 * kPts : kPts;
+    constexpr int N = POL ? 362 : 256;
+    constexpr int ROW = kHeadKPad + 1;       // odd row length: conflict-free column reads
     const int tid = threadIdx.x, lane = tid & 63;
     const int q = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r0 = rb * 32;
 
-    // the first weight fragments go out before the rows are staged
-    const float4v* wf = reinterpret_cast<const float4v*>(policy ? hp.ip_pol_wf : hp.ip1_val_wf) +
-                        (((size_t)cb * 4 + q) * (steps / 4)) * 64 + lane;
-    constexpr int AHEAD = 6;
-    float4v w[AHEAD];
+    const float4v* wf = reinterpret_cast<const float4v*>(POL ? hp.ip_pol_wf : hp.ip1_val_wf) +
+                        (((size_t)cb * 4 + q) * G) * 64 + lane;
+    float4v w[G];
 #pragma unroll
-    for (int g = 0; g < AHEAD; g++) w[g] = wf[(size_t)g * 64];
+    for (int g = 0; g < G; g++) w[g] = wf[(size_t)g * 64];
 
     // 32 rows of the layer's input: batch norm + ReLU of the raw head planes, zero padded
-    for (int i = tid; i < 32 * kpad; i += 256) {
-        const int r = i / kpad, k = i - r * kpad;
-        float x = 0.0f;
-        if (r0 + r < n && k < K) {
-            if (policy) {
-                const int pl = k >= kPts ? 1 : 0;
-                x = fmaxf(0.0f, hp.bn_pol_scale[pl] *
-                                    (pol[(size_t)(r0 + r) * 2 * kPts + k] - hp.bn_pol_mean[pl]));
-            } else {
-                x = fmaxf(0.0f, hp.bn_val_scale[0] *
-                                    (val[(size_t)(r0 + r) * kPts + k] - hp.bn_val_mean[0]));
-            }
+    const float s0 = POL ? hp.bn_pol_scale[0] : hp.bn_val_scale[0];
+    const float m0 = POL ? hp.bn_pol_mean[0] : hp.bn_val_mean[0];
+    const float s1 = POL ? hp.bn_pol_scale[1] : s0;
+    const float m1 = POL ? hp.bn_pol_mean[1] : m0;
+    constexpr int U = KP / 8;                // 32 * KP values on 256 threads: all in one go
+    for (int i0 = tid; i0 < 32 * KP; i0 += 256 * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int i = i0 + u * 256;
+            const int r = i / KP, k = i - r * KP;
+            x[u] = (i < 32 * KP && r0 + r < n && k < KK) ? src[(size_t)(r0 + r) * KK + k] : 0.0f;
         }
-        xs[r * ROW + k] = x;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int i = i0 + u * 256;
+            const int r = i / KP, k = i - r * KP;
+            const bool second = POL && k >= kPts;
+            float y = 0.0f;
+            if (r0 + r < n && k < KK)
+                y = fmaxf(0.0f, (second ? s1 : s0) * (x[u] - (second ? m1 : m0)));
+            if (i < 32 * KP) xs[r * ROW + k] = y;
+        }
     }
     __syncthreads();
 
     float16v acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.0f;
-    const float* xa = xs + (lane & 31) * ROW + q * steps * 2 + (lane >> 5);
-    const int groups = steps / 4;
-    for (int g0 = 0; g0 < groups; g0 += AHEAD) {
+    const float* xa = xs + (lane & 31) * ROW + q * STEPS * 2 + (lane >> 5);
 #pragma unroll
-        for (int u = 0; u < AHEAD; u++) {
-            const int g = g0 + u;
-            if (g < groups) {     // uniform
-                const float4v b = w[u];
-                if (g + AHEAD < groups) w[u] = wf[(size_t)(g + AHEAD) * 64];
-                const float* x = xa + g * 8;
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[0], b.x, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[2], b.y, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[4], b.z, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[6], b.w, acc, 0, 0, 0);
-            }
-        }
+    for (int g = 0; g < G; g++) {
+        const float* x = xa + g * 8;
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[0], w[g].x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[2], w[g].y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[4], w[g].z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[6], w[g].w, acc, 0, 0, 0);
     }
     __syncthreads();   // everyone is done with the staged rows: reuse them for the partial tiles
 
@@ -2480,20 +2481,29 @@ __global__ __launch_bounds__(256) void heads_fc_k(const float* __restrict__ pol,
     for (int r = 0; r < 16; r++)
         red[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 33 + (lane & 31)] = acc[r];
     __syncthreads();
-    const int N = policy ? 362 : 256;
+    const float* bias = POL ? hp.ip_pol_b : hp.ip1_val_b;
     for (int i = tid; i < 32 * 32; i += 256) {
         const int r = i >> 5, j = i & 31;
         const int col = cb * 32 + j;
         if (r0 + r < n && col < N) {
-            float v = xs[r * 33 + j] + xs[32 * 33 + r * 33 + j] + xs[2 * 32 * 33 + r * 33 + j] +
-                      xs[3 * 32 * 33 + r * 33 + j];
-            if (policy) {
-                logits[(size_t)(r0 + r) * 362 + col] = v + hp.ip_pol_b[col];
-            } else {
-                hidden[(size_t)(r0 + r) * 256 + col] = fmaxf(0.0f, v + hp.ip1_val_b[col]);
-            }
+            const float v = xs[r * 33 + j] + xs[32 * 33 + r * 33 + j] +
+                            xs[2 * 32 * 33 + r * 33 + j] + xs[3 * 32 * 33 + r * 33 + j];
+            out[(size_t)(r0 + r) * N + col] = POL ? v + bias[col] : fmaxf(0.0f, v + bias[col]);
         }
     }
+}
+
+__global__ __launch_bounds__(256) void heads_fc_k(const float* __restrict__ pol,
+                                                  const float* __restrict__ val, HeadParams hp,
+                                                  float* __restrict__ logits,
+                                                  float* __restrict__ hidden, int n) {
+    __shared__ float xs[32 * (kHeadKPad + 1)];
+    const int tasks = kHeadColsPol + kHeadColsVal;
+    const int rb = blockIdx.x / tasks, task = blockIdx.x - rb * tasks;
+    if (task < kHeadColsPol)
+        heads_fc_body<true>(xs, pol, hp, logits, task, rb * 32, n);
+    else
+        heads_fc_body<false>(xs, val, hp, hidden, task - kHeadColsPol, rb * 32, n);
 }
 
 // One wavefront per position: softmax over the logits at `temperature`, and the value
