@@ -459,10 +459,23 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const P* base, size_
 // cost twice the time (32 channels at 64 boards: 16.4 us against 12.9): they stay write-back.
 template <int CG> constexpr int xform_store_policy() { return CG == 64 ? kStoreThrough : 0; }
 constexpr int kPlane = 22;       // LDS plane: 19 points + 1 zero halo before + 2 after
+// Strides of the plane in channel pairs.  A store or load instruction of the transform
+// touches the same cell of every tile in the wavefront, CG / 2 consecutive pairs each, and
+// tiles lie 4 cells (and 4 rows) apart: with cells of exactly CG / 2 pairs the narrow shapes
+// put all their tiles on the same banks (16 channels: 8 tiles on 8 of 32 banks, measured
+// 237 k conflict cycles in 351 k active ones per launch).  Padded so that four cells and
+// four rows both advance the bank by CG / 2, consecutive tiles take consecutive groups of
+// banks (7.7 k conflict cycles left, the halo; the launch takes as long as before: LDS was
+// not what it waited for).  The 64-channel shape (one tile per 32 lanes) needs no padding.
+constexpr int plane_cell_pairs(int cg) { return cg == 16 ? 10 : cg == 32 ? 20 : cg / 2; }
+constexpr int plane_row_pairs(int cg) {
+    return cg == 16 ? kPlane * 10 + 6 : cg == 32 ? kPlane * 20 + 4 : kPlane * (cg / 2);
+}
+constexpr int plane_pairs(int cg) { return kPlane * plane_row_pairs(cg); }
 constexpr int fuse_waves(int cg) { return (kTilesPerBoard + 128 / cg - 1) / (128 / cg); }
 
 // The body of the kernel, for work-group `wg` of the launch's transform work-groups, with
-// the LDS plane handed in (kPlane * kPlane * CG / 2 channel pairs); returns the work item
+// the LDS plane handed in (plane_pairs(CG) channel pairs); returns the work item
 // (board * channel groups + channel group) it processed, or -1 if `wg` had none.
 // VPOL = cache policy of the stores of V.  VSLAB: V is written channel group by channel
 // group, [36][Kp / CG][Tp][CG], instead of [36][Tp][Kp]: the 25 tiles of this work-group's
@@ -475,6 +488,7 @@ __device__ __forceinline__ int out_in_transform_body(
     int Kp, int Tp) {
     typedef typename BufIO2<P>::pair_t pair_t;
     constexpr int CP = CG / 2;        // channel pairs per plane cell = lanes per tile
+    constexpr int CS = plane_cell_pairs(CG), RS = plane_row_pairs(CG);   // plane strides
     constexpr int TPW = 64 / CP;      // tiles per wavefront
     constexpr int WAVES = fuse_waves(CG);
     // Work-group w runs on die w % 8, each die with its own L2.  The narrow shapes share
@@ -569,18 +583,18 @@ __device__ __forceinline__ int out_in_transform_body(
             int cell;
             if (q < 3 * kPlane) {
                 const int row = q < kPlane ? 0 : (q < 2 * kPlane ? kBoard + 1 : kBoard + 2);
-                cell = row * kPlane + (q % kPlane);
+                cell = row * RS + (q % kPlane) * CS;
             } else {
                 const int e = q - 3 * kPlane, y = 1 + e / 3, c3 = e % 3;
-                cell = y * kPlane + (c3 == 0 ? 0 : kBoard + c3);
+                cell = y * RS + (c3 == 0 ? 0 : kBoard + c3) * CS;
             }
-            ybuf[cell * CP + cl] = zero;
+            ybuf[cell + cl] = zero;
         }
     }
 
     // ---- phase 1: A^T m A, BN (+ residual), ReLU -> LDS plane (+ memory)
     // plane cell of the tile's patch origin (board row 4by-1, column 4bx-1)
-    pair_t* const origin = ybuf + ((4 * by) * kPlane + 4 * bx) * CP + cl;
+    pair_t* const origin = ybuf + (4 * by) * RS + (4 * bx) * CS + cl;
     pair_t keep[16];   // this tile's activations, written to memory after the barrier
     {
         float o[2][16];
@@ -616,7 +630,7 @@ __device__ __forceinline__ int out_in_transform_body(
                 sv.y = act_to_storage<P>(fmaxf(
                     0.0f, fmaf((float)r[i * 4 + jj].y, rfac, fmaf(o[1][i * 4 + jj], sc[1], nb[1]))));
                 keep[i * 4 + jj] = sv;
-                if (valid && i < ny && jj < nx) origin[((i + 1) * kPlane + (jj + 1)) * CP] = sv;
+                if (valid && i < ny && jj < nx) origin[(i + 1) * RS + (jj + 1) * CS] = sv;
             }
         }
     }
@@ -641,7 +655,7 @@ __device__ __forceinline__ int out_in_transform_body(
 #pragma unroll
         for (int yy = 0; yy < 6; yy++)
 #pragma unroll
-            for (int xx = 0; xx < 6; xx++) raw[yy * 6 + xx] = origin[(yy * kPlane + xx) * CP];
+            for (int xx = 0; xx < 6; xx++) raw[yy * 6 + xx] = origin[yy * RS + xx * CS];
         pair_t outp[36];
 #pragma unroll
         for (int v = 0; v < 2; v++) {
@@ -689,7 +703,7 @@ __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     const P* M, const P* __restrict__ res, P* __restrict__ act_out, P* Vn,
     const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int n,
     int Kp, int Tp) {
-    __shared__ typename BufIO2<P>::pair_t ybuf[kPlane * kPlane * (CG / 2)];
+    __shared__ typename BufIO2<P>::pair_t ybuf[plane_pairs(CG)];
     (void)out_in_transform_body<P, CG, xform_store_policy<CG>()>(ybuf, blockIdx.x, M, res, act_out, Vn, bn_scale, bn_mean,
                                        rfac, n, Kp, Tp);
 }
@@ -1780,7 +1794,7 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
     unsigned n_xform_wg, unsigned long long* flags, unsigned long long epoch, unsigned* gave_up) {
     typedef BufIO2<half_t>::pair_t pair_t;
     constexpr int NKC = 2 * NW;      // tower layers: as many input as output channels
-    constexpr int XBYTES = kPlane * kPlane * (CG / 2) * (int)sizeof(pair_t);
+    constexpr int XBYTES = plane_pairs(CG) * (int)sizeof(pair_t);
     constexpr int GBYTES = gemm_stream_lds_halves<NKC, NBLK, NW>() * 2;
     // More than half of a compute unit's 160 KiB, whatever the roles need: two work-groups of
     // this launch never share a unit.  A GEMM work-group beside a transform work-group sends
