@@ -190,10 +190,11 @@ public:
         }
         m_gave_up.alloc(1);
         *m_gave_up.p = 0;
-        // measurement knob: 0 never, 1 where it pays and the forward is alone on the device,
-        // 2 always (one array), 3 always (two arrays, up to 8 boards)
+        // measurement knobs.  LZHIP_FUSE: 0 never, 1 where it pays (the default), 2 wherever a
+        // fused launch exists; LZHIP_SLAB=0: tile arrays row by row at every batch
         if (const char* e = std::getenv("LZHIP_FUSE")) m_fuse = std::atoi(e);
         if (const char* e = std::getenv("LZHIP_INPLACE")) m_in_place = std::atoi(e) != 0;
+        if (const char* e = std::getenv("LZHIP_SLAB")) m_slab = std::atoi(e) != 0;
         m_scalar.alloc(4);
         for (int i = 0; i < kTimerPool; i++) {
             HIP_CHECK(hipEventCreate(&m_ev_start[i]));
@@ -624,15 +625,37 @@ public:
         HIP_CHECK(hipMemcpy(d_sc.p, sc.data(), sizeof(float) * m_Fp, hipMemcpyHostToDevice));
         HIP_CHECK(hipMemcpy(d_mn.p, mn.data(), sizeof(float) * m_Fp, hipMemcpyHostToDevice));
         launch_in_transform<P>(a_in, ln.V.p, n, Cp, m_Tp, ln.stream, nullptr);
-        launch_gemm<P>(ln.V.p, L.U.p, L.Uf.p, ln.M.p, Tu, m_Tp, Cp, m_Fp, ln.stream, nullptr);
+        // The layout a forward of n boards keeps its tiles in: the GEMM and the output
+        // transform run as they do there.  In a forward a tower layer's V comes slab by slab
+        // from the fused transform; here the input transform's rows are re-laid on the host.
+        int slab = 0;
+        if constexpr (sizeof(P) == 2) {
+            if (m_slab && L.Uf.p != nullptr && gemm_stream_shape(Tu, Cp, m_Fp, 2))
+                slab = tile_slab(n, m_Fp, 2, true);
+        }
+        std::vector<P> v_rows;
+        if (Vout || (slab != 0 && Cp != 64)) {
+            v_rows.resize((size_t)kPos * m_Tp * Cp);
+            HIP_CHECK(hipStreamSynchronize(ln.stream));
+            HIP_CHECK(hipMemcpy(v_rows.data(), ln.V.p, v_rows.size() * sizeof(P), hipMemcpyDeviceToHost));
+        }
+        if (slab != 0 && Cp != 64) {
+            std::vector<P> g(v_rows.size());
+            for (int p = 0; p < kPos; p++)
+                for (int t = 0; t < m_Tp; t++)
+                    for (int c = 0; c < Cp; c++)
+                        g[(((size_t)p * (Cp / slab) + c / slab) * m_Tp + t) * slab + c % slab] =
+                            v_rows[((size_t)p * m_Tp + t) * Cp + c];
+            HIP_CHECK(hipMemcpy(ln.V.p, g.data(), g.size() * sizeof(P), hipMemcpyHostToDevice));
+        }
+        launch_gemm<P>(ln.V.p, L.U.p, L.Uf.p, ln.M.p, Tu, m_Tp, Cp, m_Fp, ln.stream, nullptr, slab);
         launch_out_transform<P>(ln.M.p, r, ln.act[2].p, d_sc.p, d_mn.p, 1.0f, n, m_Fp, m_Tp,
-                                ln.stream, nullptr);
+                                ln.stream, nullptr, slab);
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipStreamSynchronize(ln.stream));
         const int T = n * kTilesPerBoard;
         if (Vout) {
-            std::vector<P> h((size_t)kPos * m_Tp * Cp);
-            HIP_CHECK(hipMemcpy(h.data(), ln.V.p, h.size() * sizeof(P), hipMemcpyDeviceToHost));
+            const std::vector<P>& h = v_rows;
             for (int t = 0; t < T; t++)
                 for (int p = 0; p < kPos; p++)
                     for (int c = 0; c < C; c++)
@@ -645,8 +668,9 @@ public:
             for (int t = 0; t < T; t++)
                 for (int p = 0; p < kPos; p++)
                     for (int k = 0; k < F; k++)
-                        Mout[(((size_t)(t / 25) * kPos + p) * F + k) * 25 + t % 25] =
-                            (float)h[((size_t)p * m_Tp + t) * m_Fp + k];
+                        Mout[(((size_t)(t / 25) * kPos + p) * F + k) * 25 + t % 25] = (float)
+                            (slab != 0 ? h[(((size_t)p * (m_Fp / slab) + k / slab) * m_Tp + t) * slab + k % slab]
+                                       : h[((size_t)p * m_Tp + t) * m_Fp + k]);
         }
         if (Yout) {
             std::vector<P> h((size_t)n * kPts * m_Fp);
@@ -836,21 +860,26 @@ private:
             launch_pack_input_bits<P>(d_bits, w.act0, n, kInPlanes, m_C0p, w.stream,
                                       timer(timed, LZHIP_K_PACK));
         launch_in_transform<P>(w.act0, w.V, n, m_C0p, w.Tp, w.stream, timer(timed, LZHIP_K_IN));
-        // Small batches of fp16 towers (xform_gemm_shape; xform_gemm_pays says which of the
-        // launch's two forms, if any): the transform of layer l and the GEMM of layer l + 1 go
-        // out as one launch when this forward has the device to itself: the fused
-        // launch shortens a chain of dependent kernels (one lane, 256 filters: +17 %
-        // evaluations/s at one board, +9 % at 16), but its waiting work-groups hold compute
-        // units that another lane's kernels would otherwise use (three lanes at 8 boards:
-        // -20 %).  Both ways give the same bits.  Not under graph capture (the launch carries a number that
-        // has to differ from launch to launch), not when every launch is timed, and not on
-        // the static working memory.
-        bool fused = false, fused_two_arrays = false;
+        // Small batches of fp16 towers (xform_gemm_shape) keep their tile arrays slab by slab
+        // (tile_slab) from the first GEMM's output to the last transform's input -- nothing
+        // outside this function sees them -- and send the transform of layer l and the GEMM
+        // of layer l + 1 as one launch where xform_gemm_pays says that is faster: the fused
+        // launch shortens a chain of dependent kernels, but its waiting work-groups hold
+        // compute units that another lane's kernels could use, so the answer depends on
+        // whether this forward has the device to itself.  All ways give the same bits.  No
+        // fused launches under graph capture (the launch carries a number that has to differ
+        // from launch to launch), when every launch is timed, or on the static working memory.
+        int slab = 0;
         if constexpr (sizeof(P) == 2) {
-            const int form = m_fuse == 2 ? 1 : m_fuse == 3 ? 2 : xform_gemm_pays(n, m_Fp);
-            fused = m_fuse > 0 && form > 0 && (w.alone || m_fuse > 1) && !timed && !m_use_graph &&
-                    w.flags != nullptr && xform_gemm_shape(n, m_Fp, 2) && (form == 1 || n <= 8);
-            fused_two_arrays = form == 2;
+            if (m_slab && m_layers.size() > 1 && m_layers[1].Uf.p != nullptr &&
+                gemm_stream_shape(Tu, m_Fp, m_Fp, 2))
+                slab = tile_slab(n, m_Fp, 2, w.alone);
+        }
+        bool fused = false;
+        if constexpr (sizeof(P) == 2) {
+            fused = m_fuse > 0 && !timed && !m_use_graph && w.flags != nullptr &&
+                    xform_gemm_shape(n, m_Fp, 2) &&
+                    (m_fuse > 1 || xform_gemm_pays(n, m_Fp, slab, w.alone));
         }
         // With the streaming GEMM the tower's layers work in place: M_l is written over V_l
         // and V_{l+1} over M_l (see the kernels), so a lane's tiles are one array instead of
@@ -862,7 +891,7 @@ private:
                               m_layers[1].Uf.p != nullptr;
         int cur = 0, nxt = 1;  // block input (skip) / block output
         launch_gemm<P>(w.V, m_layers[0].U.p, m_layers[0].Uf.p, w.M, Tu, w.Tp, m_layers[0].Cp, m_Fp,
-                       w.stream, timer(timed, LZHIP_K_GEMM));
+                       w.stream, timer(timed, LZHIP_K_GEMM), slab);
         for (int l = 0; l < nl; l++) {
             Layer& L = m_layers[l];
             const bool block_end = (l % 2) == 0;      // layer 0 and second convs
@@ -870,7 +899,7 @@ private:
             P* out = l == 0 ? w.act[cur] : w.act[nxt];
             if (l == nl - 1) {
                 launch_out_transform<P>(tiles, res, out, L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp,
-                                        w.Tp, w.stream, timer(timed, LZHIP_K_OUT));
+                                        w.Tp, w.stream, timer(timed, LZHIP_K_OUT), slab);
                 launch_head_conv<P>(out, m_w3.p, m_s[nl], d_pol, d_val, n, m_Fp, w.stream,
                                     timer(timed, LZHIP_K_HEAD));
             } else {
@@ -878,20 +907,19 @@ private:
                 bool done = false;
                 if constexpr (sizeof(P) == 2) {
                     if (fused) {
-                        launch_xform_gemm(w.M, res, block_end ? out : nullptr,
-                                          fused_two_arrays ? w.V : w.M, L.d_scale.p,
+                        launch_xform_gemm(w.M, res, block_end ? out : nullptr, w.M, L.d_scale.p,
                                           L.d_mean.p, L.rfac, n, m_Fp, w.Tp, N.Uf.p, w.flags,
-                                          ++*w.epoch, m_gave_up.p, w.stream);
+                                          ++*w.epoch, m_gave_up.p, w.stream, slab);
                         done = true;
                     }
                 }
                 if (!done) {
                     launch_out_in_transform<P>(tiles, res, block_end ? out : nullptr, w.V,
                                                L.d_scale.p, L.d_mean.p, L.rfac, n, m_Fp, w.Tp,
-                                               w.stream, timer(timed, LZHIP_K_OUTIN));
+                                               w.stream, timer(timed, LZHIP_K_OUTIN), slab);
                     if (in_place) tiles = w.V;
                     launch_gemm<P>(w.V, N.U.p, N.Uf.p, tiles, Tu, w.Tp, N.Cp, m_Fp, w.stream,
-                                   timer(timed, LZHIP_K_GEMM));
+                                   timer(timed, LZHIP_K_GEMM), slab);
                 }
             }
             if (block_end && l >= 2) { const int o = cur; cur = nxt; nxt = o; }
@@ -1012,6 +1040,7 @@ private:
     bool m_use_graph = std::getenv("LZHIP_GRAPH") != nullptr;
     int m_fuse = 1;                      // fused transform + GEMM launches (see enqueue_forward)
     bool m_in_place = true;              // tower layers keep V and M in one array (see enqueue_forward)
+    bool m_slab = true;                  // small batches keep the tile arrays slab by slab (tile_slab)
     PinnedBuf<unsigned> m_gave_up;       // set by a fused launch whose wait ran into its limit
 };
 

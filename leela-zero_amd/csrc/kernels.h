@@ -55,10 +55,14 @@ template <typename P> bool gemm_supports_channels(int Cp);
 // T = real tile rows (25 per board); Tp = allocated rows, a multiple of kTileRowPad.
 // Uf: the same filters in the fragment order of the streaming kernels (see
 // build_stream_filters), or null; taken when gemm_stream_shape(T, Cp, Kp, sizeof(P)).
+// slab (0, or tile_slab's 16 / 32; streaming shapes only): M is written slab by slab,
+// [36][Kp / slab][Tp][slab], and V read that way too unless it is the first layer's (Cp == 64).
 template <typename P>
 void launch_gemm(const P* V, const P* U, const P* Uf, P* M, int T, int Tp, int Cp, int Kp,
-                 hipStream_t s, LaunchTimer* t);
+                 hipStream_t s, LaunchTimer* t, int slab = 0);
 bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes);
+// Layout of the tile arrays that suits a forward of n boards: 0 row by row, else the slab width.
+int tile_slab(int n, int Kp, int elem_bytes, bool alone);
 // src [36][C][F] fp32 (F fastest) -> dst in the operand order of the streaming kernel for
 // elements of elem_bytes (2: [36][Kp/32][Cp/16][64][8], 4: [36][Kp/32][Cp/8][64][4]), values
 // in fp32, zero padded; convert_filters turns such an array into fp16 on the device.
@@ -66,35 +70,38 @@ void build_stream_filters(const float* src, int C, int F, int Cp, int Kp, int el
                           float* dst);
 void convert_filters(const float* src, _Float16* dst, size_t n, hipStream_t s);
 
-// M [36][Tp][Kp] -> out [n][361][Kp]:  max(0, scale*(A^T m A - mean) + rfac*res)
+// M [36][Tp][Kp] (slab > 0: [36][Kp / slab][Tp][slab]) -> out [n][361][Kp]:
+// max(0, scale*(A^T m A - mean) + rfac*res)
 template <typename P>
 void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scale,
                           const float* bn_mean, float rfac, int n, int Kp, int Tp,
-                          hipStream_t s, LaunchTimer* t);
+                          hipStream_t s, LaunchTimer* t, int slab = 0);
 
 // Output transform of one layer fused with the input transform of the next:
 // M [36][Tp][Kp] -> V_next [36][Tp][Kp]; the activation [n][361][Kp] is also
-// written to act_out unless that is null.  Needs Kp to be a multiple of 64.
+// written to act_out unless that is null.  Needs Kp to be a multiple of 64.  slab (0, 16 or
+// 32): both tile arrays lie slab by slab and a work-group takes `slab` channels.
 template <typename P>
 void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
                              const float* bn_mean, float rfac, int n, int Kp, int Tp,
-                             hipStream_t s, LaunchTimer* t);
+                             hipStream_t s, LaunchTimer* t, int slab = 0);
 
 // launch_out_in_transform of one layer and launch_gemm of the next (filters Uf, in the
 // streaming kernel's order) as one launch, for the shapes xform_gemm_shape accepts (fp16;
-// 256 filters up to 32 boards, 192 up to 42, 128 up to 64).  M is read by the transform and rewritten by the GEMM.
+// 256 filters up to 32 boards, 192 up to 42, 128 up to 64).  M is read by the transform and
+// rewritten by the GEMM; V is M (row by row: slab = 0) or M or a second array (slab by slab).
 // flags: kFusedFlagsPerBoard 64-bit words per board (zero before the first launch); epoch: a
 // value no earlier launch on these flags used; *gave_up is set to 1 if a wait inside the
 // launch ran into its limit (the results are then invalid).
 constexpr int kFusedFlagsPerBoard = 16;
 bool xform_gemm_shape(int n, int Kp, int elem_bytes);
-// Which form is the faster way for a forward that is alone on the device (measured): 0 none,
-// 1 V and M one array (launch_xform_gemm with V == M), 2 two arrays (V != M, up to 8 boards).
-int xform_gemm_pays(int n, int Kp);
+// Whether the fused launch is the faster way (measured) for a forward of n boards with the tile
+// arrays in slabs of `slab` channels (0: rows) that has the device to itself or not.
+bool xform_gemm_pays(int n, int Kp, int slab, bool alone);
 void launch_xform_gemm(_Float16* M, const _Float16* res, _Float16* act_out, _Float16* V,
                        const float* bn_scale, const float* bn_mean, float rfac, int n, int Kp,
                        int Tp, const _Float16* Uf, unsigned long long* flags,
-                       unsigned long long epoch, unsigned* gave_up, hipStream_t s);
+                       unsigned long long epoch, unsigned* gave_up, hipStream_t s, int slab = 0);
 
 // 1x1 head convolutions: act [n][361][Cp] x w[3][Cp] -> pol [n][2][361], val [n][361],
 // both multiplied by out_scale.

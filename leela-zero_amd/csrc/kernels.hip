@@ -253,7 +253,7 @@ template <typename P>
 __global__ __launch_bounds__(256) void out_transform_k(
     const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ out,
     const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int T,
-    int Kp, int Tp) {
+    int Kp, int Tp, int slab) {
     constexpr int VN = ChanVec<P>::N;
     const int lpt = Kp / VN;
     const int gid = blockIdx.x * 256 + threadIdx.x;
@@ -265,7 +265,9 @@ __global__ __launch_bounds__(256) void out_transform_k(
     const int by = j / 5, bx = j - by * 5;
 
     float m[VN][36];
-    const P* msrc = M + (size_t)t * Kp + c;
+    // slab > 0: M lies slab by slab, [36][Kp / slab][Tp][slab]
+    const P* msrc = slab > 0 ? M + ((size_t)(c / slab) * Tp + t) * slab + c % slab
+                             : M + (size_t)t * Kp + c;
     const size_t pstride = (size_t)Tp * Kp;
 #pragma unroll
     for (int p = 0; p < 36; p++) {
@@ -333,11 +335,13 @@ __global__ __launch_bounds__(256) void out_transform_k(
 template <typename P>
 void launch_out_transform(const P* M, const P* res, P* out, const float* bn_scale,
                           const float* bn_mean, float rfac, int n, int Kp, int Tp,
-                          hipStream_t s, LaunchTimer* t) {
+                          hipStream_t s, LaunchTimer* t, int slab) {
     const int T = n * kTilesPerBoard;
     const int lanes = T * (Kp / ChanVec<P>::N);
+    if (slab != 0 && (slab % ChanVec<P>::N != 0 || Kp % slab != 0))
+        throw std::invalid_argument("out_transform: slab width does not fit");
     launch(out_transform_k<P>, dim3((lanes + 255) / 256), dim3(256), s, t, M, res, out,
-           bn_scale, bn_mean, rfac, T, Kp, Tp);
+           bn_scale, bn_mean, rfac, T, Kp, Tp, slab);
 }
 
 // ---------------------------------------------------------------------------
@@ -477,11 +481,11 @@ constexpr int fuse_waves(int cg) { return (kTilesPerBoard + 128 / cg - 1) / (128
 // The body of the kernel, for work-group `wg` of the launch's transform work-groups, with
 // the LDS plane handed in (plane_pairs(CG) channel pairs); returns the work item
 // (board * channel groups + channel group) it processed, or -1 if `wg` had none.
-// VPOL = cache policy of the stores of V.  VSLAB: V is written channel group by channel
-// group, [36][Kp / CG][Tp][CG], instead of [36][Tp][Kp]: the 25 tiles of this work-group's
-// board and channel group are then one contiguous run per Winograd position (whole lines,
-// which is what makes write-through stores cheap), for a consumer that knows (xform_gemm_k).
-template <typename P, int CG, int VPOL, bool VSLAB = false>
+// VPOL = cache policy of the stores of V.  VSLAB / MSLAB: V is written / M is read channel
+// group by channel group, [36][Kp / CG][Tp][CG], instead of [36][Tp][Kp] (tile_slab): the 25
+// tiles of this work-group's board and channel group are then one contiguous run per
+// Winograd position (whole lines, which is also what makes write-through stores cheap).
+template <typename P, int CG, int VPOL, bool VSLAB = false, bool MSLAB = false>
 __device__ __forceinline__ int out_in_transform_body(
     typename BufIO2<P>::pair_t* ybuf, unsigned wg, const P* M, const P* res, P* act_out, P* Vn,
     const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int n,
@@ -545,12 +549,18 @@ __device__ __forceinline__ int out_in_transform_body(
     // for it.  The scheduling barrier keeps the compiler from sinking those loads behind
     // the first arithmetic on M.
     pair_t m[36];   // as stored; converted where used
+    // the same two offsets in the slab layout, [36][Kp / CG][Tp][CG]
+    unsigned voff_s = cl * 2 * esz + (valid ? sub : 0u) * (unsigned)CG * esz;
+    asm volatile("" : "+v"(voff_s));
+    const unsigned soff_s =
+        ((unsigned)cg * (unsigned)Tp + (unsigned)(b * kTilesPerBoard + TPW * wave)) *
+        (unsigned)CG * esz;
 #pragma unroll
     for (int xx = 0; xx < 6; xx++) {
-        unsigned so = soff_t + (unsigned)xx * pstride;
+        unsigned so = (MSLAB ? soff_s : soff_t) + (unsigned)xx * pstride;
 #pragma unroll
         for (int row = 0; row < 6; row++) {
-            m[row * 6 + xx] = BufIO2<P>::load_raw(rM, voff_t, so);
+            m[row * 6 + xx] = BufIO2<P>::load_raw(rM, MSLAB ? voff_s : voff_t, so);
             so += 6u * pstride;
         }
         __builtin_amdgcn_sched_barrier(0);   // keep the columns in this order
@@ -679,12 +689,7 @@ __device__ __forceinline__ int out_in_transform_body(
         }
         LZ_STAMP(4);
         if (valid) {
-            unsigned so = soff_t, vo = voff_t;
-            if constexpr (VSLAB) {
-                vo = cl * 2 * esz + sub * (unsigned)CG * esz;
-                so = ((unsigned)cg * (unsigned)Tp + (unsigned)(b * kTilesPerBoard + TPW * wave)) *
-                     (unsigned)CG * esz;
-            }
+            unsigned so = VSLAB ? soff_s : soff_t, vo = VSLAB ? voff_s : voff_t;
 #pragma unroll
             for (int p = 0; p < 36; p++) {
                 BufIO2<P>::template store<VPOL>(outp[p], rV, vo, so);
@@ -698,20 +703,23 @@ __device__ __forceinline__ int out_in_transform_body(
 
 // M and Vn may be one array (every value of M is in a register before the same lane writes
 // the value of V that takes its place), so neither is declared free of aliases.
-template <typename P, int CG>
+// SLAB: M and V lie slab by slab, [36][Kp / CG][Tp][CG] (see tile_slab); V's stores are then
+// whole lines and go out write-through.
+template <typename P, int CG, bool SLAB = false>
 __global__ __launch_bounds__(fuse_waves(CG) * 64) void out_in_transform_k(
     const P* M, const P* __restrict__ res, P* __restrict__ act_out, P* Vn,
     const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int n,
     int Kp, int Tp) {
     __shared__ typename BufIO2<P>::pair_t ybuf[plane_pairs(CG)];
-    (void)out_in_transform_body<P, CG, xform_store_policy<CG>()>(ybuf, blockIdx.x, M, res, act_out, Vn, bn_scale, bn_mean,
-                                       rfac, n, Kp, Tp);
+    (void)out_in_transform_body<P, CG, SLAB ? kStoreThrough : xform_store_policy<CG>(), SLAB,
+                                SLAB>(ybuf, blockIdx.x, M, res, act_out, Vn, bn_scale, bn_mean,
+                                      rfac, n, Kp, Tp);
 }
 
 template <typename P>
 void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const float* bn_scale,
                              const float* bn_mean, float rfac, int n, int Kp, int Tp,
-                             hipStream_t s, LaunchTimer* t) {
+                             hipStream_t s, LaunchTimer* t, int slab) {
     // With few boards a narrow shape spreads a board's arithmetic over more compute units;
     // the 64-channel shape moves whole lines.  Measured at 256 filters with the layers working
     // in place (transform + GEMM per layer, us, with 16 / 32 / 64 channels per work-group):
@@ -722,7 +730,15 @@ void launch_out_in_transform(const P* M, const P* res, P* act_out, P* Vn, const 
     // of it (16 channels at batch 16: 11.2 us per launch against 7.7).
     const int items64 = n * (Kp / 64);
     auto grid = [](int items) { return dim3((unsigned)(8 * ((items + 7) / 8))); };
-    if (items64 > 80)
+    if (slab == 16)
+        launch(out_in_transform_k<P, 16, true>, grid(items64 * 4), dim3(fuse_waves(16) * 64), s,
+               t, M, res, act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
+    else if (slab == 32)
+        launch(out_in_transform_k<P, 32, true>, grid(items64 * 2), dim3(fuse_waves(32) * 64), s,
+               t, M, res, act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
+    else if (slab != 0)
+        throw std::invalid_argument("out_in_transform: slabs are 16 or 32 channels wide");
+    else if (items64 > 80)
         launch(out_in_transform_k<P, 64>, grid(items64), dim3(fuse_waves(64) * 64), s, t, M, res,
                act_out, Vn, bn_scale, bn_mean, rfac, n, Kp, Tp);
     else if (items64 > 64)
@@ -1505,8 +1521,10 @@ template <int NKC, int NBLK, int NW> constexpr int gemm_stream_lds_halves() {
 }
 
 // FUSED: the work-group is part of a fused launch (xform_gemm_k): it waits for the producers
-// of its rows, and reads V in the layout they write, [Kp / SLAB][Tp][SLAB] per position.
-template <int NKC, int NBLK, int NW, bool FUSED, int SLAB = 0>
+// of its rows.  VSLAB / MSLAB > 0: V is read / M is written slab by slab,
+// [Kp / SLAB][Tp][SLAB] per position, instead of row by row, [Tp][Kp] (the layout the narrow
+// transform shapes work in, where a work-group's 25 tiles are one contiguous run).
+template <int NKC, int NBLK, int NW, bool FUSED, int VSLAB = 0, int MSLAB = 0>
 __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg, const half_t* V,
                                                       const half_t* __restrict__ Uf, half_t* M,
                                                       int T, int Tp, int Kp, int chunks,
@@ -1526,6 +1544,10 @@ __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg,
     constexpr int OROW = CW + 8;                 // row of the output copy (halves)
     constexpr int OSTAGE = 32 * OROW;
     static_assert(NKC % 2 == 0 && D == 2, "pipeline shape");
+    constexpr int SLAB = VSLAB;
+    static_assert((VSLAB == 0 || VSLAB == 16 || VSLAB == 32) &&
+                      (MSLAB == 0 || MSLAB == 16 || MSLAB == 32),
+                  "slab widths");
 
     constexpr int NST = NBLK < 3 ? NBLK : 3;     // stages of the ring in use
     static_assert(NST * STAGE + 2 * OSTAGE == gemm_stream_lds_halves<NKC, NBLK, NW>(), "LDS size");
@@ -1585,7 +1607,7 @@ __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg,
             if (lval[i]) {
                 if constexpr (SLAB > 0)
                     st[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
-                        rV, lslab[i] + (unsigned)row * (unsigned)(SLAB * 2), 0, 16);
+                        rV, lslab[i] + (unsigned)row * (unsigned)(SLAB * 2), 0, FUSED ? 16 : 0);
                 else if constexpr (FUSED)
                     st[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
                         rV, (unsigned)(row * Cp + lcc[i] * 8) * 2u, 0, 16);
@@ -1655,20 +1677,28 @@ __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg,
     // offset outside it and are dropped by the hardware, so the stores are unconditional
     // straight-line code (a branch around them would make the compiler wait for every
     // outstanding load behind it).
-    const size_t m_bytes = (size_t)T * Kp * sizeof(half_t);
+    const size_t m_bytes = (size_t)(MSLAB > 0 ? Tp : T) * Kp * sizeof(half_t);
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(M + (size_t)p * Tp * Kp, m_bytes);
     const unsigned m_rowb = (unsigned)Kp * 2u;
     // The 32 x CW result leaves in 16-byte pieces, two per thread.  Eight wavefronts:
     // wavefront w sends rows 4w..4w+3, two whole 512-byte rows per store instruction.  Fewer:
     // the pieces are dealt to the threads in memory order (a row holds CW / 8 of them), so
     // that a store instruction still writes one contiguous KiB when the tile is the whole row.
+    // Slabs: a slab's share of the block (32 rows x MSLAB channels) is contiguous, and the
+    // pieces are dealt in that order, so a store instruction again writes one contiguous KiB.
     constexpr int PPR = CW / 8;
     auto send_rows = [&](int s) {
         const half_t* O = obuf + (s & 1) * OSTAGE;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             int r, cc;
-            if constexpr (NW == 8) {
+            if constexpr (MSLAB > 0) {
+                constexpr int PR = MSLAB / 8;              // pieces per row of a slab
+                const int piece = tid + i * NT;
+                const int g = piece / (32 * PR), rem = piece - g * (32 * PR);
+                r = rem / PR;
+                cc = g * PR + (rem - r * PR);
+            } else if constexpr (NW == 8) {
                 r = wave * 4 + hh + 2 * i;
                 cc = jrow;
             } else {
@@ -1678,8 +1708,16 @@ __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg,
             }
             const int4v v = *reinterpret_cast<const int4v*>(O + r * OROW + cc * 8);
             const unsigned row = (unsigned)((blk0 + s) * 32 + r);
-            const unsigned vo =
-                s < nreal ? row * m_rowb + (unsigned)(tn * CW + cc * 8) * 2u : 0x7ffffff0u;
+            unsigned vo;
+            if constexpr (MSLAB > 0) {
+                constexpr int PR = MSLAB / 8;
+                const unsigned slab = (unsigned)(tn * (CW / MSLAB) + cc / PR);
+                vo = (s < nreal && row < (unsigned)T)
+                         ? ((slab * (unsigned)Tp + row) * (unsigned)MSLAB + (unsigned)(cc % PR) * 8u) * 2u
+                         : 0x7ffffff0u;
+            } else {
+                vo = s < nreal ? row * m_rowb + (unsigned)(tn * CW + cc * 8) * 2u : 0x7ffffff0u;
+            }
             __builtin_amdgcn_raw_buffer_store_b128(v, rM, vo, 0, kStoreThrough);
         }
     };
@@ -1743,15 +1781,15 @@ __device__ __forceinline__ void wino_gemm_stream_body(half_t* smem, unsigned wg,
 // V and M may be one array when the tile is the whole row of M (tiles_n == 1, as many input
 // as output channels): a work-group has a block of V in LDS before it writes the block of M
 // that takes its place, and no other work-group touches those rows.
-template <int NKC, int NBLK, int NW>
+template <int NKC, int NBLK, int NW, int VSLAB = 0, int MSLAB = 0>
 __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* V,
                                                           const half_t* __restrict__ Uf,
                                                           half_t* M, int T, int Tp,
                                                           int Kp, int chunks, int nblk_total,
                                                           int tiles_n, int seg) {
     __shared__ __attribute__((aligned(16))) half_t smem[gemm_stream_lds_halves<NKC, NBLK, NW>()];
-    wino_gemm_stream_body<NKC, NBLK, NW, false>(smem, blockIdx.x, V, Uf, M, T, Tp, Kp, chunks,
-                                                nblk_total, tiles_n, seg, StreamWait{});
+    wino_gemm_stream_body<NKC, NBLK, NW, false, VSLAB, MSLAB>(
+        smem, blockIdx.x, V, Uf, M, T, Tp, Kp, chunks, nblk_total, tiles_n, seg, StreamWait{});
 }
 
 // ---------------------------------------------------------------------------
@@ -1779,14 +1817,12 @@ __global__ __launch_bounds__(64 * NW) void wino_gemm_stream_k(const half_t* V,
 //
 // The buffers: the transform reads M and writes V, the GEMM reads V and writes M -- the
 // same M.  A GEMM work-group writes rows of M only after every transform work-group of
-// the boards those rows belong to has finished, i.e. after their last read.  Two forms:
-//   SLABV = false: V and M are one array in M's layout, each stage overwriting its input
-//     (as the separate launches do); the written-through 32- and 64-byte pieces of V then
-//     land in lines this die's L2 already holds.  The form for 14 boards and more.
-//   SLABV = true: V is a second array, laid out channel group by channel group
-//     ([36][Kp / CG][Tp][CG], see out_in_transform_body; nothing outside the launch reads
-//     it), so that the transform writes whole lines.  The faster form at 1 to 6 boards.
-template <int CG, int NBLK, int NW, bool SLABV>
+// the boards those rows belong to has finished, i.e. after their last read.  V and M are
+// normally one array, each stage overwriting its input, as the separate launches do.
+// SLAB: both lie slab by slab, [36][Kp / CG][Tp][CG] (tile_slab), so that the transform reads
+// and writes whole lines; row by row, its written-through 32- and 64-byte pieces of V land in
+// lines that the die's L2 already holds from reading M.
+template <int CG, int NBLK, int NW, bool SLAB>
 __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) void xform_gemm_k(
     half_t* M, const half_t* res, half_t* act_out, half_t* V, const float* __restrict__ bn_scale,
     const float* __restrict__ bn_mean, float rfac, int n, int Kp, int Tp,
@@ -1808,7 +1844,7 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
     LZ_STAMP(0);
     if (blockIdx.x < n_xform_wg) {
         if (wave >= fuse_waves(CG)) return;    // the block is sized for the larger role
-        const int item = out_in_transform_body<half_t, CG, kStoreThrough, SLABV>(
+        const int item = out_in_transform_body<half_t, CG, kStoreThrough, SLAB, SLAB>(
             reinterpret_cast<pair_t*>(lds), blockIdx.x, M, res, act_out, V, bn_scale, bn_mean,
             rfac, n, Kp, Tp);
         if (item < 0) return;                  // uniform over the work-group
@@ -1822,7 +1858,7 @@ __global__ __launch_bounds__(64 * (NW > fuse_waves(CG) ? NW : fuse_waves(CG))) v
         LZ_STAMP(7);
     } else {
         if (wave >= NW) return;
-        wino_gemm_stream_body<NKC, NBLK, NW, true, SLABV ? CG : 0>(
+        wino_gemm_stream_body<NKC, NBLK, NW, true, SLAB ? CG : 0, SLAB ? CG : 0>(
             reinterpret_cast<half_t*>(lds), blockIdx.x - n_xform_wg, V, Uf, M, T, Tp, Kp, chunks,
             nblk_total, tiles_n, seg, StreamWait{flags, epoch, gave_up, Kp / CG});
     }
@@ -2076,7 +2112,7 @@ bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes) {
 
 template <int NKC, int NW>
 static void launch_gemm_stream_nkc(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
-                                   int Kp, hipStream_t s, LaunchTimer* t) {
+                                   int Kp, hipStream_t s, LaunchTimer* t, int slab) {
     const int nblk = (T + 31) / 32;
     const int nb = gemm_stream_blocks(T, Kp);
     const int chunks = (nblk + nb - 1) / nb;
@@ -2085,32 +2121,80 @@ static void launch_gemm_stream_nkc(const half_t* V, const half_t* Uf, half_t* M,
     int seg = (n_items + 7) / 8;
     seg = (seg + tiles_n - 1) / tiles_n * tiles_n;
     const dim3 grid(8 * seg), block(64 * NW);
-    switch (nb) {
-        case 1: launch(wino_gemm_stream_k<NKC, 1, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        case 2: launch(wino_gemm_stream_k<NKC, 2, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        case 4: launch(wino_gemm_stream_k<NKC, 4, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        case 8: launch(wino_gemm_stream_k<NKC, 8, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
-        default: launch(wino_gemm_stream_k<NKC, 16, NW>, grid, block, s, t, V, Uf, M, T, Tp, Kp, chunks, nblk, tiles_n, seg); break;
+#define LZ_STREAM(NB, VS, MS)                                                                     \
+    launch(wino_gemm_stream_k<NKC, NB, NW, VS, MS>, grid, block, s, t, V, Uf, M, T, Tp, Kp,      \
+           chunks, nblk, tiles_n, seg)
+    // slabs: the first layer reads its 64 input planes row by row (NKC == 4) and writes slabs;
+    // the pairs (slab width, blocks per work-group) are those tile_slab hands out
+    constexpr bool FIRST = NKC == 4;
+    if (slab == 16) {
+        switch (nb) {
+            case 1: LZ_STREAM(1, FIRST ? 0 : 16, 16); return;
+            case 2: LZ_STREAM(2, FIRST ? 0 : 16, 16); return;
+            case 4: LZ_STREAM(4, FIRST ? 0 : 16, 16); return;
+            default: break;
+        }
+    } else if (slab == 32) {
+        switch (nb) {
+            case 2: LZ_STREAM(2, FIRST ? 0 : 32, 32); return;
+            case 4: LZ_STREAM(4, FIRST ? 0 : 32, 32); return;
+            case 8: LZ_STREAM(8, FIRST ? 0 : 32, 32); return;
+            default: break;
+        }
     }
+    if (slab != 0) throw std::invalid_argument("no slab-layout GEMM instantiated for this batch");
+    switch (nb) {
+        case 1: LZ_STREAM(1, 0, 0); break;
+        case 2: LZ_STREAM(2, 0, 0); break;
+        case 4: LZ_STREAM(4, 0, 0); break;
+        case 8: LZ_STREAM(8, 0, 0); break;
+        default: LZ_STREAM(16, 0, 0); break;
+    }
+#undef LZ_STREAM
 }
 
 // NW = Kp / 32 wavefronts per work-group; the first layer reads the 64 padded input planes.
 template <int NW>
 static void launch_gemm_stream_nw(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
-                                  int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
+                                  int Cp, int Kp, hipStream_t s, LaunchTimer* t, int slab) {
     if (Cp == 64)
-        launch_gemm_stream_nkc<4, NW>(V, Uf, M, T, Tp, Kp, s, t);
+        launch_gemm_stream_nkc<4, NW>(V, Uf, M, T, Tp, Kp, s, t, slab);
     else
-        launch_gemm_stream_nkc<2 * NW, NW>(V, Uf, M, T, Tp, Kp, s, t);
+        launch_gemm_stream_nkc<2 * NW, NW>(V, Uf, M, T, Tp, Kp, s, t, slab);
 }
 
 static void launch_gemm_stream(const half_t* V, const half_t* Uf, half_t* M, int T, int Tp,
-                               int Cp, int Kp, hipStream_t s, LaunchTimer* t) {
+                               int Cp, int Kp, hipStream_t s, LaunchTimer* t, int slab) {
     switch (Kp) {
-        case 256: launch_gemm_stream_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
-        case 192: launch_gemm_stream_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
-        default: launch_gemm_stream_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t); break;
+        case 256: launch_gemm_stream_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t, slab); break;
+        case 192: launch_gemm_stream_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t, slab); break;
+        default: launch_gemm_stream_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t, slab); break;
     }
+}
+
+// The layout of the tile arrays for a forward of n boards: 0 = row by row, [36][Tp][Kp];
+// 16 or 32 = slab by slab, [36][Kp / w][Tp][w], for the batches that take the transform
+// shapes of that many channels per work-group (fp16 towers of 128, 192 and 256 filters).  A
+// transform work-group (one board, w channels) then reads and writes its 25 tiles as one
+// contiguous run of 25 w values per Winograd position instead of 25 pieces of 2 w bytes, and
+// the GEMM reads and writes a slab's share of a 32-row block as one contiguous run: the same
+// bytes in a quarter (an eighth) of the requests to the L2s.  Measured, transform alone at
+// 256 filters, rows / slabs: 16 boards 7.0 / 6.0 us, 24 boards 9.2 (64-channel shape) / 7.3,
+// 32 boards 9.3 / 7.8; from 40 boards the 64-channel shape (whole lines anyway) is level.
+// Forwards, evaluations/s, rows -> slabs (best launch form each):
+//   40x256 one lane: 1 board +6 %, 4 +10 %, 8 +9 %, 12 +8 %, 16 +10 %, 20 +2 %, 24 +3 %,
+//          28 +6 %, 32 +6 %; three lanes: 12 +8 %, 16 +5 %, 20 +4 %, 24 -8 %, 28 -3 %, 32 -2 %
+//   15x192 one lane: 1 to 4 +8 %, 8 +12 %, 16 +15 %, 21 +16 %, 26 +3 %, 32 +8 %, 42 0 %;
+//          three lanes: 8 and 12 -3 %, 16 0 % (two lanes +13 %), 21 +11 %, 26 +14 %, 42 +4 %
+//   10x128 one lane: 1 to 8 +3..6 %, 16 +10 %, 24 +8 %, 32 +15 %, 40 +4 %, 48 0 %, 64 -1 %;
+//          three lanes: 16 -1 % (two lanes +9 %), 32 +2 %, 40 +8 %, 48 0 %, two lanes at 64 -5 %
+// hence: every such batch at 192 filters, up to 44 boards at 128, and at 256 filters up to
+// 20 boards, or up to 32 when the forward has the device to itself (`alone`).
+int tile_slab(int n, int Kp, int elem_bytes, bool alone) {
+    if (!xform_gemm_shape(n, Kp, elem_bytes)) return 0;
+    if (Kp == 256 && n > 20 && !alone) return 0;
+    if (Kp == 128 && n > 44) return 0;
+    return n * (Kp / 64) <= 64 ? 16 : 32;
 }
 
 // Shapes served by the fused transform + GEMM launch: fp16 towers of 128, 192 and 256
@@ -2121,28 +2205,32 @@ bool xform_gemm_shape(int n, int Kp, int elem_bytes) {
            n * (Kp / 64) <= 128;
 }
 
-// Which form of the fused launch, if any, is the faster way to run a forward that has the
-// device to itself: 0 none (separate launches), 1 one array, 2 two arrays.  Measured on one
-// lane (40x256 / 15x192 / 10x128, evaluations per second against separate launches, which
-// also work in place):
-//   256 filters  two arrays +17 % at 1 board, +9 % at 2, +6 % at 4, +3 % at 6 (one array
-//                +10, +9, +3, +3 %), both -4..-7 % at 8; one array -1..-3 % at 10 to 14,
-//                +8 % at 16, +5 % at 20, +9 % at 24, +3 % at 32
-//   192 filters  neither form up to 20 boards (-3..-11 %); one array +7 % at 24, +10 % at
-//                32, +19 % at 42
-//   128 filters  neither form up to 24 boards (-3..-12 %); one array +5 % at 32, +3 % at
-//                42, +8 % at 48, +25 % at 64
-// The one-array form pays where the transform's work-groups fill the device, so that GEMM
-// work-groups start as those retire instead of after a hand-over between launches; the
-// two-array form where a few boards leave most of the device to GEMM work-groups that fetch
-// their filters (128 KiB each at 256 filters) while the transform runs.
-int xform_gemm_pays(int n, int Kp) {
-    if (Kp == 256) return n <= 6 ? 2 : n >= 16 ? 1 : 0;
-    if (Kp == 192) return n >= 22 ? 1 : 0;
-    return n >= 32 ? 1 : 0;
+// Whether the fused launch is the faster way to run a forward of n boards whose tile arrays
+// lie in slabs of `slab` channels (0: row by row), with the device to itself (`alone`) or
+// shared with other lanes' forwards.  Measured (40x256 / 15x192 / 10x128, evaluations per
+// second against separate launches):
+//   alone, slabs: the launch pays where the transform's work-groups fill the device in one
+//     round (n Kp / slab between 232 and 256), so that GEMM work-groups, which have fetched
+//     their filters meanwhile, start as those retire instead of after a hand-over between
+//     launches: 256 filters +3 % at 16 and 32 boards, 192 filters +4 % at 21 and +6 % at 42,
+//     128 filters +5 % at 32; elsewhere -1..-10 % (256 filters: 8 to 12 boards -3..-6 %, 24
+//     and 28 -4 %).  And at 256 filters up to 7 boards, where most of the device is free for
+//     GEMM work-groups that fetch 128 KiB of filters each while the transform runs: +16 % at
+//     1 board, +14 % at 2, +10 % at 3 and 4, +6 % at 5, +2 % at 6 (192 and 128 filters have a
+//     half and a quarter of those bytes to hide: 0..-7 % up to 8 boards).
+//   not alone, slabs: with few boards the device is mostly idle, and a lane's waiting GEMM
+//     work-groups take nothing from the other lanes: three lanes, 256 filters +35 % at 3
+//     boards, +19 % at 5, 0 % at 6, -17 % at 8; 192 filters +72 % at 1, +46 % at 2, +54 % at 4,
+//     +12 % at 8, +3 % at 12, -10 % at 16; 128 filters +55 % at 1 to 4, +10 % at 8, -14 % at 16.
+//   rows (what is left of them: 128 filters from 49 boards, alone): +8 % at 48, +25 % at 64.
+bool xform_gemm_pays(int n, int Kp, int slab, bool alone) {
+    if (slab == 0) return alone && Kp == 128 && n >= 32;
+    if (!alone) return n <= (Kp == 256 ? 5 : Kp == 192 ? 10 : 8);
+    const int groups = n * (Kp / slab);
+    return (groups >= 232 && groups <= 256) || (Kp == 256 && n <= 7);
 }
 
-template <int CG, int NBLK, int NW, bool SLABV>
+template <int CG, int NBLK, int NW, bool SLAB>
 static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, half_t* V,
                                  const float* bn_scale, const float* bn_mean, float rfac, int n,
                                  int Kp, int Tp, const half_t* Uf, unsigned long long* flags,
@@ -2154,7 +2242,7 @@ static void launch_xform_gemm_as(half_t* M, const half_t* res, half_t* act_out, 
     const int seg = (kPos * chunks * tiles_n + 7) / 8;
     const unsigned n_xform_wg = 8u * (unsigned)((n * (Kp / CG) + 7) / 8);
     constexpr int WAVES = NW > fuse_waves(CG) ? NW : fuse_waves(CG);
-    hipLaunchKernelGGL((xform_gemm_k<CG, NBLK, NW, SLABV>),
+    hipLaunchKernelGGL((xform_gemm_k<CG, NBLK, NW, SLAB>),
                        dim3(n_xform_wg + 8u * (unsigned)seg), dim3(64 * WAVES), 0, s, M, res,
                        act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, T, chunks, nblk, tiles_n,
                        seg, n_xform_wg, flags, epoch, gave_up);
@@ -2164,19 +2252,28 @@ template <int NW>
 static void launch_xform_gemm_nw(half_t* M, const half_t* res, half_t* act_out, half_t* V,
                                  const float* bn_scale, const float* bn_mean, float rfac, int n,
                                  int Kp, int Tp, const half_t* Uf, unsigned long long* flags,
-                                 unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
+                                 unsigned long long epoch, unsigned* gave_up, hipStream_t s,
+                                 int slab) {
     const int nb = gemm_stream_blocks(n * kTilesPerBoard, Kp);
     const bool narrow = n * (Kp / 64) <= 64;     // 16-channel transform groups, else 32
-#define LZ_FUSED(CG, NB, SLABV)                                                                   \
-    launch_xform_gemm_as<CG, NB, NW, SLABV>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp,   \
-                                            Tp, Uf, flags, epoch, gave_up, s)
-    if (V != M) {   // the second array: the few-board form
-        if (narrow && nb == 1) LZ_FUSED(16, 1, true);
-        else throw std::invalid_argument("the two-array fused launch serves up to 8 boards");
-        return;
-    }
+#define LZ_FUSED(CG, NB, SLAB)                                                                  \
+    launch_xform_gemm_as<CG, NB, NW, SLAB>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp,    \
+                                           Tp, Uf, flags, epoch, gave_up, s)
     // the pairs that occur: 16-channel groups up to 64 / (Kp / 64) boards, i.e. up to 7, 14 or
     // (128 filters) 25 blocks of 32 rows per position; 32-channel groups up to twice that
+    if (slab != 0) {   // both arrays slab by slab (they may be one)
+        if (slab != (narrow ? 16 : 32))
+            throw std::invalid_argument("fused launch: the slab width follows the batch");
+        if (narrow && nb == 1) LZ_FUSED(16, 1, true);
+        else if (narrow && nb == 2) LZ_FUSED(16, 2, true);
+        else if (narrow && nb == 4) LZ_FUSED(16, 4, true);
+        else if (!narrow && nb == 2) LZ_FUSED(32, 2, true);
+        else if (!narrow && nb == 4) LZ_FUSED(32, 4, true);
+        else if (!narrow && nb == 8) LZ_FUSED(32, 8, true);
+        else throw std::invalid_argument("no fused launch instantiated for this batch");
+        return;
+    }
+    if (V != M) throw std::invalid_argument("fused launch: row by row, V and M are one array");
     if (narrow && nb == 1) LZ_FUSED(16, 1, false);
     else if (narrow && nb == 2) LZ_FUSED(16, 2, false);
     else if (narrow && nb == 4) LZ_FUSED(16, 4, false);
@@ -2187,18 +2284,18 @@ static void launch_xform_gemm_nw(half_t* M, const half_t* res, half_t* act_out, 
 #undef LZ_FUSED
 }
 
-// V == M: the one-array form; V != M: the two-array form (up to 8 boards).
+// slab: 0 (V and M one array, row by row) or tile_slab's width (slab by slab; one array or two).
 // flags: kFusedFlagsPerBoard words per board of the largest batch, zero before the first
 // launch; epoch: a number no earlier launch on these flags has used (grows by one per launch).
 void launch_xform_gemm(half_t* M, const half_t* res, half_t* act_out, half_t* V,
                        const float* bn_scale, const float* bn_mean, float rfac, int n, int Kp,
                        int Tp, const half_t* Uf, unsigned long long* flags,
-                       unsigned long long epoch, unsigned* gave_up, hipStream_t s) {
+                       unsigned long long epoch, unsigned* gave_up, hipStream_t s, int slab) {
     if (!xform_gemm_shape(n, Kp, 2)) throw std::invalid_argument("no fused launch for this shape");
     switch (Kp) {
-        case 256: launch_xform_gemm_nw<8>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s); break;
-        case 192: launch_xform_gemm_nw<6>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s); break;
-        default: launch_xform_gemm_nw<4>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s); break;
+        case 256: launch_xform_gemm_nw<8>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s, slab); break;
+        case 192: launch_xform_gemm_nw<6>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s, slab); break;
+        default: launch_xform_gemm_nw<4>(M, res, act_out, V, bn_scale, bn_mean, rfac, n, Kp, Tp, Uf, flags, epoch, gave_up, s, slab); break;
     }
 }
 
@@ -2229,7 +2326,8 @@ static void launch_gemm_stream32_nw(const float* V, const float* Uf, float* M, i
 }
 
 static void launch_gemm_stream(const float* V, const float* Uf, float* M, int T, int Tp, int Cp,
-                               int Kp, hipStream_t s, LaunchTimer* t) {
+                               int Kp, hipStream_t s, LaunchTimer* t, int slab) {
+    if (slab != 0) throw std::invalid_argument("the fp32 GEMM works row by row");
     if (Kp == 256)
         launch_gemm_stream32_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t);
     else
@@ -2272,13 +2370,14 @@ template bool gemm_supports_channels<half_t>(int);
 // must be a multiple of 256.
 template <typename P>
 void launch_gemm(const P* V, const P* U, const P* Uf, P* M, int T, int Tp, int Cp, int Kp,
-                 hipStream_t s, LaunchTimer* t) {
+                 hipStream_t s, LaunchTimer* t, int slab) {
     constexpr int BK = 128 / (int)sizeof(P);
     const int nk = Cp / BK;
     if (Uf != nullptr && gemm_stream_shape(T, Cp, Kp, (int)sizeof(P))) {
-        launch_gemm_stream(V, Uf, M, T, Tp, Cp, Kp, s, t);
+        launch_gemm_stream(V, Uf, M, T, Tp, Cp, Kp, s, t, slab);
         return;
     }
+    if (slab != 0) throw std::invalid_argument("only the streaming GEMM works slab by slab");
     // The 256 x 256 tile pays off once its tiles can occupy most of the 256 compute units
     // (measured at 256 filters: from 6 row tiles = 216 work-groups, batch 52; with 5 = 180 the
     // 128 x 128 tiles are 2 % ahead; fp32 keeps the earlier hand-over at 160).
@@ -2582,12 +2681,13 @@ void launch_heads(const float* pol, const float* val, HeadParams hp, float tempe
     template void launch_in_transform<P>(const P*, P*, int, int, int, hipStream_t,             \
                                          LaunchTimer*);                                        \
     template void launch_gemm<P>(const P*, const P*, const P*, P*, int, int, int, int,         \
-                                 hipStream_t, LaunchTimer*);                                   \
+                                 hipStream_t, LaunchTimer*, int);                              \
     template void launch_out_transform<P>(const P*, const P*, P*, const float*, const float*,  \
-                                          float, int, int, int, hipStream_t, LaunchTimer*);    \
+                                          float, int, int, int, hipStream_t, LaunchTimer*,     \
+                                          int);                                                \
     template void launch_out_in_transform<P>(const P*, const P*, P*, P*, const float*,         \
                                              const float*, float, int, int, int, hipStream_t,  \
-                                             LaunchTimer*);                                    \
+                                             LaunchTimer*, int);                               \
     template void launch_head_conv<P>(const P*, const float*, float, float*, float*, int, int, \
                                       hipStream_t, LaunchTimer*);                              \
     template void launch_absmax<P>(const P*, size_t, float*, hipStream_t);

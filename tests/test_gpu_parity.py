@@ -30,15 +30,18 @@ def make_pipes(pkg, netgen, orc, blocks, filters, seed, precision, max_batch):
 
 
 @pytest.mark.parametrize("precision", [0, 1])
-@pytest.mark.parametrize("filters,n", [(8, 3), (64, 3), (192, 3), (128, 3), (128, 40), (256, 3),
-                                       (256, 40)])
+@pytest.mark.parametrize("filters,n", [(8, 3), (64, 3), (192, 3), (192, 30), (128, 3), (128, 40),
+                                       (256, 3), (256, 16), (256, 20), (256, 40)])
 def test_single_layer_stages(pkg, netgen, orc, precision, filters, n):
     """V, M and Y of one convolution layer against the oracle's stages, for the input
     layer (18 planes) and a residual-tower layer with a skip connection.  The M stage is
     the check the reference's tuner makes of every GEMM it times, against a plain sgemm
     (reference src/Tuner.cpp:262-301); 128 and 256 filters put the streaming GEMMs of both
     storage types under it, at 3 boards (one 32-row block per work-group) and at 40 (several
-    blocks per work-group, a last block of 8 rows)."""
+    blocks per work-group, a last block of 8 rows).  The fp16 GEMM and output transform run
+    in the layout a forward of that many boards keeps its tiles in: slabs of 16 channels at
+    3 and 16 boards, of 32 at 20 (256 filters), 30 (192) and 40 (128), rows at 40 boards of
+    256 filters."""
     print("case: single_layer precision=%d filters=%d n=%d" % (precision, filters, n), flush=True)
     net, pipe, ref, _ = make_pipes(pkg, netgen, orc, 1, filters, 40 + filters, precision,
                                    max(4, n))
@@ -541,48 +544,57 @@ def test_graph_replays_match_stream_launches(pkg, netgen, orc):
 def test_fused_launches_match_separate_launches(pkg, netgen, orc, filters, maxb, batches):
     """An fp16 tower of 128, 192 or 256 filters sends the transform of a layer and the GEMM of
     the next as one launch where that is faster and the forward has the device to itself, up
-    to the batch where the transform changes to its 64-channel shape.  Handles that always fuse
-    with V and M in one array (LZHIP_FUSE=2), that fuse with two arrays up to 8 boards (3),
-    that never fuse (0) and that decide per forward (the default) must give the same bits, at batches
-    that take each of the fused shapes (1, 2, 4 or 8 blocks of 32 rows per GEMM work-group,
-    16- or 32-channel transform groups), on one lane and with all lanes busy; and the result
-    agrees with the oracle."""
+    to the batch where the transform changes to its 64-channel shape, and up to that batch it
+    keeps its tile arrays slab by slab instead of row by row.  Handles that always fuse
+    (LZHIP_FUSE=2), that never fuse (0) and that decide per forward (the default), each with
+    the slab layout and (LZHIP_SLAB=0) without,
+    must give the same bits, at batches that take each of the shapes (1, 2, 4 or 8 blocks of 32
+    rows per GEMM work-group, 16- or 32-channel transform groups), on one lane and with all
+    lanes busy; and the result agrees with the oracle."""
     import os
     import torch
     print("case: fused launches, %d filters" % filters, flush=True)
     pipes = {}
-    for mode in ("2", "3", "0", None):
-        if mode is None:
-            os.environ.pop("LZHIP_FUSE", None)
-        else:
-            os.environ["LZHIP_FUSE"] = mode
-        try:
-            net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 4, filters, 3100, pkg.FP16, maxb)
-        finally:
-            os.environ.pop("LZHIP_FUSE", None)
-        pipes[mode] = pipe
+    for slab in ("0", None):
+        for mode in ("2", "0", None):
+            for key, v in (("LZHIP_FUSE", mode), ("LZHIP_SLAB", slab)):
+                if v is None:
+                    os.environ.pop(key, None)
+                else:
+                    os.environ[key] = v
+            try:
+                net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 4, filters, 3100, pkg.FP16, maxb)
+            finally:
+                os.environ.pop("LZHIP_FUSE", None)
+                os.environ.pop("LZHIP_SLAB", None)
+            pipes[(mode, slab)] = pipe
     x = netgen.synthetic_inputs(maxb, seed=3101)
+    base = pipes[("0", "0")]                      # separate launches, row layout
     for n in batches:
-        want = pipes["0"].forward_batch(x[:n])
-        for mode in ("2", "3", None):
-            got = pipes[mode].forward_batch(x[:n])
-            assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), (n, mode)
+        want = base.forward_batch(x[:n])
+        for key, pipe in pipes.items():
+            if pipe is base:
+                continue
+            got = pipe.forward_batch(x[:n])
+            assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), (n, key)
     rp, rv = ref.forward(x[7])
     nb = batches[4]
-    want = pipes["0"].forward_batch(x[:nb])
+    want = base.forward_batch(x[:nb])
     assert rel_l2(want[0][7], rp) <= 2e-2 and rel_l2(want[1][7], rv) <= 2e-2
     # every lane at once, many forwards in a row without synchronisation, always fused
-    pipe = pipes["2"]
     d_in = torch.from_numpy(x).cuda()
-    outs = [(torch.zeros(nb, 722, device="cuda"), torch.zeros(nb, 361, device="cuda"))
-            for _ in range(pipe.lanes())]
-    torch.cuda.synchronize()
-    for rep in range(8):
-        for k, (pol, val) in enumerate(outs):
-            pipe.forward_batch_device(nb, d_in.data_ptr(), pol.data_ptr(), val.data_ptr(), lane=k)
-    pipe.sync()
-    for pol, val in outs:
-        assert np.array_equal(pol.cpu().numpy(), want[0]) and np.array_equal(val.cpu().numpy(), want[1])
+    for key in (("2", None), ("2", "0"), ("0", None)):
+        pipe = pipes[key]
+        outs = [(torch.zeros(nb, 722, device="cuda"), torch.zeros(nb, 361, device="cuda"))
+                for _ in range(pipe.lanes())]
+        torch.cuda.synchronize()
+        for rep in range(8):
+            for k, (pol, val) in enumerate(outs):
+                pipe.forward_batch_device(nb, d_in.data_ptr(), pol.data_ptr(), val.data_ptr(), lane=k)
+        pipe.sync()
+        for pol, val in outs:
+            assert np.array_equal(pol.cpu().numpy(), want[0]), key
+            assert np.array_equal(val.cpu().numpy(), want[1]), key
     for pipe in pipes.values():
         pipe.close()
 
