@@ -537,9 +537,9 @@ def test_graph_replays_match_stream_launches(pkg, netgen, orc):
 
 
 @pytest.mark.parametrize("filters,maxb,batches", [
-    (256, 32, (1, 5, 8, 9, 16, 17, 23, 32)),
+    (256, 32, (1, 5, 8, 9, 16, 17, 20, 21, 23, 32)),
     (192, 42, (1, 7, 10, 15, 21, 22, 37, 42)),
-    (128, 64, (1, 8, 9, 18, 32, 33, 36, 64)),
+    (128, 64, (1, 8, 9, 18, 32, 33, 36, 44, 45, 64)),
 ])
 def test_fused_launches_match_separate_launches(pkg, netgen, orc, filters, maxb, batches):
     """An fp16 tower of 128, 192 or 256 filters sends the transform of a layer and the GEMM of
