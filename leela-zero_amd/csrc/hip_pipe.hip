@@ -291,9 +291,11 @@ public:
             L.Cp = l == 0 ? m_C0p : m_Fp;
             tmp.assign((size_t)kPos * m_Fp * L.Cp, 0.0f);
             // One copy of the filters, in the order the GEMM of this width and precision
-            // reads them.  Whether that is the streaming kernel does not depend on the
-            // batch, so a network holds either the fragment order or the row order, never both.
-            if (gemm_stream_shape(kTilesPerBoard, L.Cp, m_Fp, (int)sizeof(P))) {
+            // reads them.  Whether that is the streaming kernel does not depend on the batch
+            // of a forward (only on the handle's limit), so a network holds either the
+            // fragment order or the row order, never both.
+            if (gemm_stream_shape(kTilesPerBoard, L.Cp, m_Fp, (int)sizeof(P)) &&
+                gemm_stream_prefers(m_Fp, (int)sizeof(P), m_max_batch)) {
                 build_stream_filters(U[l], L.C, F, L.Cp, m_Fp, (int)sizeof(P), tmp.data());
                 upload(L.Uf);
             } else {

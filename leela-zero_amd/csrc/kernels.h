@@ -61,6 +61,9 @@ template <typename P>
 void launch_gemm(const P* V, const P* U, const P* Uf, P* M, int T, int Tp, int Cp, int Kp,
                  hipStream_t s, LaunchTimer* t, int slab = 0);
 bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes);
+// Whether a handle for batches up to max_batch should hold the streaming kernels' filters
+// where gemm_stream_shape allows them (measured; see there).
+bool gemm_stream_prefers(int Kp, int elem_bytes, int max_batch);
 // Layout of the tile arrays that suits a forward of n boards: 0 row by row, else the slab width.
 int tile_slab(int n, int Kp, int elem_bytes, bool alone);
 // src [36][C][F] fp32 (F fastest) -> dst in the operand order of the streaming kernel for

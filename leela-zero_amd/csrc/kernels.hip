@@ -2096,18 +2096,24 @@ static StreamSplit gemm_stream_split(int T, int Kp) {
     return {chunks, nb};
 }
 
-// Whether launch_gemm takes a streaming kernel for this shape (the caller then has to hold
-// the fragment-order filters): input layer (64 padded planes) and tower layers, any batch, of
-// fp16 nets of 128, 192 and 256 filters (one column tile of Kp / 32 wavefronts; at 64 filters
-// the tiled kernel is as fast: 3.0 against 3.5 us at 4 boards, 3.5 against 3.5 at 33) and of
-// fp32 nets of 128 and 256 filters (64 boards, 256 filters: 88 -> 79-83 us per launch, 48
-// boards 78 -> 58, 8 boards 22 -> 13; 128 filters: 27 -> 23 at 64 boards).  fp32 at 192 filters
-// stays with the tiled kernel: six wavefronts sit unevenly on four SIMDs and it is ahead from
-// 24 boards (26.4 against 28.2 us; 16 boards 20.0 against 17.0), and one kernel family per
-// network keeps a position's result independent of the batch it is evaluated in.
+// Whether launch_gemm takes a streaming kernel for this shape when it is handed the
+// fragment-order filters: input layer (64 padded planes) and tower layers, any batch, of nets
+// of 128, 192 and 256 filters in both storage types (one column tile of Kp / 32 wavefronts;
+// at 64 filters the tiled kernel is as fast: 3.0 against 3.5 us at 4 boards, 3.5 against 3.5 at
+// 33).  fp32, tiled -> streaming: 256 filters 88 -> 79-83 us per launch at 64 boards, 78 -> 58 at
+// 48, 22 -> 13 at 8; 128 filters 27 -> 23 at 64 boards.  At 192 filters in fp32 six wavefronts
+// sit unevenly on four SIMDs: the streaming kernel is ahead up to 24 boards on one lane (15x192
+// forwards +6 % at 1 board, +11 % at 8, +20 % at 16, +10 % at 24; all lanes +4 % at 8, +2 % at 16,
+// -15 % at 24) and behind beyond (-4 % at 32, -8 % at 64): gemm_stream_prefers says which kernel
+// family a handle of a given batch limit holds the filters for.  One family per handle keeps a
+// position's result independent of the batch it is evaluated in.
 bool gemm_stream_shape(int T, int Cp, int Kp, int elem_bytes) {
+    (void)elem_bytes;
     if (T < 1 || !(Cp == 64 || Cp == Kp)) return false;
-    return Kp == 128 || Kp == 256 || (Kp == 192 && elem_bytes == 2);
+    return Kp == 128 || Kp == 256 || Kp == 192;
+}
+bool gemm_stream_prefers(int Kp, int elem_bytes, int max_batch) {
+    return !(Kp == 192 && elem_bytes == 4 && max_batch > 16);
 }
 
 template <int NKC, int NW>
@@ -2330,6 +2336,8 @@ static void launch_gemm_stream(const float* V, const float* Uf, float* M, int T,
     if (slab != 0) throw std::invalid_argument("the fp32 GEMM works row by row");
     if (Kp == 256)
         launch_gemm_stream32_nw<8>(V, Uf, M, T, Tp, Cp, Kp, s, t);
+    else if (Kp == 192)
+        launch_gemm_stream32_nw<6>(V, Uf, M, T, Tp, Cp, Kp, s, t);
     else
         launch_gemm_stream32_nw<4>(V, Uf, M, T, Tp, Cp, Kp, s, t);
 }

@@ -348,12 +348,13 @@ def test_handle_created_from_a_weights_file(pkg, netgen, orc, tmp_path):
 
 
 @pytest.mark.parametrize("precision", [0, 1])
-@pytest.mark.parametrize("filters,maxb", [(64, 8), (128, 40), (192, 40), (256, 40)])
+@pytest.mark.parametrize("filters,maxb", [(64, 8), (128, 40), (192, 16), (192, 40), (256, 40)])
 def test_batch_composition_does_not_change_results(pkg, netgen, orc, precision, filters, maxb):
     """A position evaluated alone, in a partial batch and in a full batch gives
     bit-identical planes: rows of the GEMM are independent, and a network's layers run one
     kernel family at every batch (whatever the tile shapes, blocks per work-group or channel
-    groups the batch selects, a value is summed in the same order)."""
+    groups the batch selects, a value is summed in the same order).  fp32 at 192 filters takes
+    the streaming GEMM in handles of up to 16 positions and the tiled one in larger ones."""
     print("case: batch composition %d filters precision=%d" % (filters, precision), flush=True)
     net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 2, filters, 77, precision, maxb)
     x = netgen.synthetic_inputs(maxb, seed=5)
