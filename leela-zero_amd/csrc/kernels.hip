@@ -2227,11 +2227,12 @@ bool xform_gemm_shape(int n, int Kp, int elem_bytes) {
 //   not alone, slabs: with few boards the device is mostly idle, and a lane's waiting GEMM
 //     work-groups take nothing from the other lanes: three lanes, 256 filters +35 % at 3
 //     boards, +19 % at 5, 0 % at 6, -17 % at 8; 192 filters +72 % at 1, +46 % at 2, +54 % at 4,
-//     +12 % at 8, +3 % at 12, -10 % at 16; 128 filters +55 % at 1 to 4, +10 % at 8, -14 % at 16.
-//   rows (what is left of them: 128 filters from 49 boards, alone): +8 % at 48, +25 % at 64.
+//     +12 % at 8, -10 % at 16; 128 filters +55 % at 1 to 4, +10 % at 8, -14 % at 16; two lanes
+//     the same up to 4 or 5 boards (+7..37 %) and -1..-10 % at 8: taken up to 5 (256) or 6 boards.
+//   rows (what is left of them: 128 filters from 45 boards, alone): +8 % at 48, +25 % at 64.
 bool xform_gemm_pays(int n, int Kp, int slab, bool alone) {
     if (slab == 0) return alone && Kp == 128 && n >= 32;
-    if (!alone) return n <= (Kp == 256 ? 5 : Kp == 192 ? 10 : 8);
+    if (!alone) return n <= (Kp == 256 ? 5 : 6);
     const int groups = n * (Kp / slab);
     return (groups >= 232 && groups <= 256) || (Kp == 256 && n <= 7);
 }
