@@ -1039,7 +1039,11 @@ private:
     int m_timer_class[kTimerPool] = {};
     int m_timer_used = 0;
     LaunchTimer m_timer;
-    bool m_use_graph = std::getenv("LZHIP_GRAPH") != nullptr;
+    // LZHIP_GRAPH=1 (any value but 0): forwards replay a captured graph
+    bool m_use_graph = [] {
+        const char* e = std::getenv("LZHIP_GRAPH");
+        return e != nullptr && std::atoi(e) != 0;
+    }();
     int m_fuse = 1;                      // fused transform + GEMM launches (see enqueue_forward)
     bool m_in_place = true;              // tower layers keep V and M in one array (see enqueue_forward)
     bool m_slab = true;                  // small batches keep the tile arrays slab by slab (tile_slab)
