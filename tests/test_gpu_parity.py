@@ -600,6 +600,48 @@ def test_fused_launches_match_separate_launches(pkg, netgen, orc, filters, maxb,
         pipe.close()
 
 
+def test_random_batches_on_all_lanes_match_the_plain_forward(pkg, netgen, orc):
+    """A seeded sequence of 400 forwards of random batches (1 to 32 boards, 256 filters) dealt to
+    random lanes with no synchronisation between them -- so that consecutive forwards of a lane
+    change between the slab widths and the row layout, between fused and separate launches,
+    and between having the device alone and sharing it -- gives, forward by forward, the bits
+    of a handle that never fuses and keeps its tiles row by row."""
+    import os
+    import torch
+    print("case: random batches on all lanes", flush=True)
+    maxb = 32
+    os.environ["LZHIP_FUSE"] = "0"
+    os.environ["LZHIP_SLAB"] = "0"
+    try:
+        net, plain, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 256, 3300, pkg.FP16, maxb)
+    finally:
+        os.environ.pop("LZHIP_FUSE", None)
+        os.environ.pop("LZHIP_SLAB", None)
+    net, pipe, ref, h_ref = make_pipes(pkg, netgen, orc, 3, 256, 3300, pkg.FP16, maxb)
+    x = netgen.synthetic_inputs(maxb, seed=3301)
+    want = {}
+    rng = np.random.default_rng(3302)
+    plan = [(int(rng.integers(1, maxb + 1)), int(rng.integers(0, pipe.lanes()))) for _ in range(400)]
+    for n, _ in plan:
+        if n not in want:
+            want[n] = plain.forward_batch(x[:n])
+    d_in = torch.from_numpy(x).cuda()
+    outs = [(torch.zeros(maxb, 722, device="cuda"), torch.zeros(maxb, 361, device="cuda"))
+            for _ in plan]
+    torch.cuda.synchronize()
+    for i, (n, lane) in enumerate(plan):
+        pipe.forward_batch_device(n, d_in.data_ptr(), outs[i][0].data_ptr(), outs[i][1].data_ptr(),
+                                  lane=lane)
+        if i % 97 == 96:
+            pipe.sync()           # now and then a forward finds the device empty
+    pipe.sync()
+    for i, (n, lane) in enumerate(plan):
+        assert np.array_equal(outs[i][0].cpu().numpy()[:n], want[n][0]), (i, n, lane)
+        assert np.array_equal(outs[i][1].cpu().numpy()[:n], want[n][1]), (i, n, lane)
+    pipe.close()
+    plain.close()
+
+
 def test_error_behaviour_on_device(pkg, netgen):
     """Calls out of order and arguments out of range are refused with an error code and a
     message, never executed: forward before push_weights, push_weights twice, an even layer
