@@ -179,8 +179,10 @@ void launch_pack_input_bits(const uint32_t* bits, P* act, int n, int C, int Cp, 
 // lanes own consecutive channels, so every load and store of a wave covers a
 // contiguous run of the channels-last arrays.  The 6x6 patch starts one point
 // above/left of board point (4by, 4bx); points off the board read as zero.
+// (At most four wavefronts per SIMD are asked for: aiming at eight, the compiler keeps the
+// kernel within 64 registers by waiting for each of the 36 loads before it issues the next.)
 template <typename P>
-__global__ __launch_bounds__(256) void in_transform_k(const P* __restrict__ act,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void in_transform_k(const P* __restrict__ act,
                                                       P* __restrict__ V, int T, int Cp,
                                                       int Tp) {
     constexpr int VN = ChanVec<P>::N;
@@ -250,7 +252,10 @@ void launch_in_transform(const P* act, P* V, int n, int Cp, int Tp, hipStream_t 
 // out = max(0, scale*(y - mean) + rfac*res); rfac carries the ratio of the
 // activation scales of the skip connection and of this layer (1 in fp32).
 template <typename P>
-__global__ __launch_bounds__(256) void out_transform_k(
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const P* base, size_t bytes);
+
+template <typename P>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 3))) void out_transform_k(
     const P* __restrict__ M, const P* __restrict__ res, P* __restrict__ out,
     const float* __restrict__ bn_scale, const float* __restrict__ bn_mean, float rfac, int T,
     int Kp, int Tp, int slab) {
@@ -297,6 +302,8 @@ __global__ __launch_bounds__(256) void out_transform_k(
         mn[v] = bn_mean[c + v];
     }
     const size_t bbase = (size_t)b * kPts * Kp + c;
+    const __amdgpu_buffer_rsrc_t rO =
+        make_rsrc(out, (size_t)((T + kTilesPerBoard - 1) / kTilesPerBoard) * kPts * Kp * sizeof(P));
     float r[VN][16];
     if (res != nullptr) {  // uniform; clamped addresses keep the 16 loads free of branches
 #pragma unroll
@@ -326,8 +333,22 @@ __global__ __launch_bounds__(256) void out_transform_k(
             for (int v = 0; v < VN; v++)
                 val[v] = act_clamp<P>(
                     fmaxf(0.0f, sc[v] * (o[v][i * 4 + jj] - mn[v]) + rfac * r[v][i * 4 + jj]));
-            if (y < kBoard && x < kBoard)
-                ChanVec<P>::store(out + bbase + (size_t)(y * kBoard + x) * Kp, val);
+            // Unconditional store through a buffer descriptor: points off the board get an
+            // offset outside it and are dropped by the hardware (a branch around each store
+            // makes the compiler wait for the store before it).
+            const unsigned off = (y < kBoard && x < kBoard)
+                                     ? (unsigned)((bbase + (size_t)(y * kBoard + x) * Kp) * sizeof(P))
+                                     : 0xfffffff0u;
+            if constexpr (sizeof(P) == 4) {
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val[0]), rO, off,
+                                                      0, 0);
+            } else {
+                half2v h;
+                h.x = (half_t)fminf(fmaxf(val[0], -65504.0f), 65504.0f);
+                h.y = (half_t)fminf(fmaxf(val[1], -65504.0f), 65504.0f);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, h), rO, off, 0,
+                                                      0);
+            }
         }
     }
 }
